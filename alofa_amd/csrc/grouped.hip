@@ -32,7 +32,7 @@ struct GroupedShape {
   int x_by_slot;                        // listed: the input row is the slot itself (row_in only says which slots are in use)
   int tiles, tiles_per_batch;           // tiles in all; dense: row tiles of a batch (0: listed)
   int64_t gate_stride;                  // kGrSigmoidGate: gate[row, batch * out_batch_step + o]
-  float limit, limit_last, slope;       // kGrClampedGlu
+  float limit, limit_last, slope, offset;       // kGrClampedGlu: a sigmoid(slope a) (b + offset)
 };
 
 // Every lane issues every load (from the operand's first bytes where its own are not wanted) and what is not wanted is cleared
@@ -183,7 +183,7 @@ __global__ void __launch_bounds__(256) grouped_product_kernel(TO* __restrict__ o
         } else if constexpr (kGlu) {
           const float a = fminf(y, lim);
           const float b = fminf(fmaxf(acc2[t][c][i], -lim), lim);
-          y = weight * (a * (1.f / (1.f + __expf(-s.slope * a))) * (b + 1.f));
+          y = weight * (a * (1.f / (1.f + __expf(-s.slope * a))) * (b + s.offset));
         }
         store_f32(dst + o, y);
       }
@@ -312,7 +312,7 @@ __global__ void __launch_bounds__(256) grouped_tiled_kernel(TO* __restrict__ out
         } else if constexpr (kGlu) {
           const float a = fminf(y, lim);
           const float b = fminf(fmaxf(acc[t][c + 2][i], -lim), lim);
-          y = weight * (a * (1.f / (1.f + __expf(-s.slope * a))) * (b + 1.f));
+          y = weight * (a * (1.f / (1.f + __expf(-s.slope * a))) * (b + s.offset));
         }
         store_f32(dst + o, y);
       }
@@ -340,7 +340,8 @@ __global__ void __launch_bounds__(1024) expert_rows_kernel(const int32_t* __rest
   for (int i = threadIdx.x; i < tiles; i += 1024) tile_batch[i] = -1;
   __syncthreads();
   const int pairs = T * top;
-  for (int i = threadIdx.x; i < pairs; i += 1024) atomicAdd(&count[chosen[i]], 1);
+  for (int i = threadIdx.x; i < pairs; i += 1024)
+    if (chosen[i] >= 0 && chosen[i] < experts) atomicAdd(&count[chosen[i]], 1);      // (a choice beyond the experts with matrices takes no slot)
   __syncthreads();
   if (threadIdx.x == 0) {
     int at = 0;
@@ -355,6 +356,10 @@ __global__ void __launch_bounds__(1024) expert_rows_kernel(const int32_t* __rest
     for (int t = first[e] / pad; t < first[e + 1] / pad; ++t) tile_batch[t] = e;
   for (int i = threadIdx.x; i < pairs; i += 1024) {
     const int e = chosen[i];
+    if (e < 0 || e >= experts) {
+      slot_of[i] = -1;
+      continue;
+    }
     const int slot = first[e] + atomicAdd(&cursor[e], 1);
     row_in[slot] = i / top;
     slot_weight[slot] = weights[i];
@@ -373,14 +378,20 @@ __global__ void __launch_bounds__(1024) expert_rows_kernel(const int32_t* __rest
 
 // ---- residual[t, c] += scale[c] * sum_k y[slot_of[t, k], c], k ascending (then the shared expert's) --------------
 __global__ void __launch_bounds__(256) experts_sum_kernel(float* __restrict__ residual, const float* __restrict__ y, const int32_t* __restrict__ slot_of,
-                                                          const float* __restrict__ scale, int T, int width, int top, int shared) {
+                                                          const float* __restrict__ scale, int T, int width, int top, int shared,
+                                                          const float* __restrict__ pass_weight, const bf16_t* __restrict__ pass_x, int64_t pass_stride, int assign) {
   const int64_t idx = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
   if (idx >= static_cast<int64_t>(T) * width) return;
   const int t = static_cast<int>(idx / width), c = static_cast<int>(idx % width);
   float sum = 0.f;
-  for (int k = 0; k < top; ++k) sum += y[static_cast<int64_t>(slot_of[t * top + k]) * width + c];
+  for (int k = 0; k < top; ++k) {
+    const int slot = slot_of[t * top + k];
+    if (slot >= 0) sum += y[static_cast<int64_t>(slot) * width + c];      // (-1: a choice without a slot)
+  }
   if (shared) sum += y[static_cast<int64_t>(slot_of[T * top + t]) * width + c];
-  residual[idx] += scale ? scale[c] * sum : sum;
+  if (pass_weight) sum += pass_weight[t] * bf16_to_f32(pass_x[static_cast<int64_t>(t) * pass_stride + c]);      // (the row itself, handed on with a weight)
+  if (scale) sum *= scale[c];
+  residual[idx] = assign ? sum : residual[idx] + sum;
 }
 
 }  // namespace alofa
@@ -422,7 +433,7 @@ static int launch_grouped(void* out, const void* x, const void* W, const void* W
 extern "C" int alofa_grouped_product(void* out, int out_dtype, int64_t out_stride, int64_t out_batch_step, const void* x, int64_t x_stride, int64_t x_batch_step,
                                      const void* W, const void* W2, int64_t w_stride, int64_t w_batch_step, int n_out, int K, int last_batch, int n_out_last,
                                      int K_last, int rows, int x_by_slot, int tiles, int tiles_per_batch, int tile_rows, const int32_t* tile_batch, const int32_t* row_in, const void* gate,
-                                     int64_t gate_stride, const float* slot_weight, float limit, float limit_last, float slope, int epilogue, hipStream_t stream) {
+                                     int64_t gate_stride, const float* slot_weight, float limit, float limit_last, float slope, float offset, int epilogue, hipStream_t stream) {
   ALOFA_REQUIRE(n_out > 0 && K > 0 && rows >= 0 && tiles >= 0, "grouped_product: bad sizes (n_out=%d K=%d rows=%d tiles=%d)", n_out, K, rows, tiles);
   ALOFA_REQUIRE(K % 8 == 0 && K_last % 8 == 0 && x_stride % 8 == 0 && x_batch_step % 8 == 0 && w_stride % 8 == 0 && w_batch_step % 8 == 0 &&
                     reinterpret_cast<uintptr_t>(x) % 16 == 0 && reinterpret_cast<uintptr_t>(W) % 16 == 0 && (W2 == nullptr || reinterpret_cast<uintptr_t>(W2) % 16 == 0),
@@ -433,7 +444,7 @@ extern "C" int alofa_grouped_product(void* out, int out_dtype, int64_t out_strid
   ALOFA_REQUIRE(epilogue != kGrClampedGlu || (W2 && out_dtype == kBF16), "grouped_product: the GLU epilogue needs a second matrix and writes bfloat16");
   if (rows == 0 || tiles == 0) return 0;
   GroupedShape s{out_stride, out_batch_step, x_stride, x_batch_step, w_stride, w_batch_step, n_out, K, last_batch, n_out_last, K_last, rows, x_by_slot, tiles, tiles_per_batch,
-                 gate_stride, limit, limit_last, slope};
+                 gate_stride, limit, limit_last, slope, offset};
   if (epilogue == kGrStore && out_dtype == kBF16) return launch_grouped<kGrStore, bf16_t>(out, x, W, W2, tile_batch, row_in, gate, slot_weight, s, tile_rows, stream);
   if (epilogue == kGrStore && out_dtype == kF32) return launch_grouped<kGrStore, float>(out, x, W, W2, tile_batch, row_in, gate, slot_weight, s, tile_rows, stream);
   if (epilogue == kGrSigmoidGate && out_dtype == kBF16) return launch_grouped<kGrSigmoidGate, bf16_t>(out, x, W, W2, tile_batch, row_in, gate, slot_weight, s, tile_rows, stream);
@@ -452,9 +463,10 @@ extern "C" int alofa_expert_rows(const int32_t* chosen, const float* weights, in
   return check_launch("expert_rows");
 }
 
-extern "C" int alofa_experts_sum(float* residual, const float* y, const int32_t* slot_of, const float* scale, int T, int width, int top, int shared, hipStream_t stream) {
+extern "C" int alofa_experts_sum(float* residual, const float* y, const int32_t* slot_of, const float* scale, int T, int width, int top, int shared,
+                                 const float* pass_weight, const void* pass_x, int64_t pass_stride, int assign, hipStream_t stream) {
   ALOFA_REQUIRE(T >= 0 && width > 0 && top > 0, "experts_sum: bad sizes");
   if (T == 0) return 0;
-  experts_sum_kernel<<<static_cast<unsigned>((static_cast<int64_t>(T) * width + 255) / 256), 256, 0, stream>>>(residual, y, slot_of, scale, T, width, top, shared);
+  experts_sum_kernel<<<static_cast<unsigned>((static_cast<int64_t>(T) * width + 255) / 256), 256, 0, stream>>>(residual, y, slot_of, scale, T, width, top, shared, pass_weight, static_cast<const bf16_t*>(pass_x), pass_stride, assign);
   return check_launch("experts_sum");
 }

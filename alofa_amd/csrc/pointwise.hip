@@ -39,19 +39,64 @@ __global__ void __launch_bounds__(256) layernorm_kernel(TO* __restrict__ out, co
   }
 }
 
+// residual[r] += layer norm of x[r] (weight, bias): the norm behind a sub-layer, on its way into the stream.
+template <typename Acc>
+__global__ void __launch_bounds__(256) layernorm_add_kernel(float* __restrict__ residual, const float* __restrict__ x, const float* __restrict__ w,
+                                                            const float* __restrict__ b, int width, float eps) {
+  __shared__ Acc scratch[4];
+  const int r = blockIdx.x;
+  const float* src = x + static_cast<int64_t>(r) * width;
+  float* dst = residual + static_cast<int64_t>(r) * width;
+  Acc s = 0;
+  for (int c = threadIdx.x; c < width; c += 256) s += static_cast<Acc>(src[c]);
+  const Acc mean = block_sum<Acc, 256>(s, scratch) / static_cast<Acc>(width);
+  Acc ss = 0;
+  for (int c = threadIdx.x; c < width; c += 256) {
+    const Acc d = static_cast<Acc>(src[c]) - mean;
+    ss += d * d;
+  }
+  const Acc var = block_sum<Acc, 256>(ss, scratch) / static_cast<Acc>(width);
+  const Acc inv = static_cast<Acc>(1) / sqrt(var + static_cast<Acc>(eps));
+  for (int c = threadIdx.x; c < width; c += 256) {
+    const Acc y = (static_cast<Acc>(src[c]) - mean) * inv * static_cast<Acc>(w[c]) + static_cast<Acc>(b[c]);
+    dst[c] = static_cast<float>(static_cast<Acc>(dst[c]) + y);
+  }
+}
+
+// out[t, c] += w[t] * x[t, c]: a row handed on with a weight of its own (float rows out, rows of any type in).
+template <typename T, typename Acc>
+__global__ void __launch_bounds__(256) add_row_scaled_kernel(float* __restrict__ out, const T* __restrict__ x, int64_t x_stride, const float* __restrict__ w,
+                                                             int64_t rows, int width) {
+  const int64_t idx = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+  if (idx >= rows * width) return;
+  const int64_t r = idx / width;
+  const float wr = w[r];
+  if (wr == 0.f) return;
+  out[idx] = static_cast<float>(static_cast<Acc>(out[idx]) + static_cast<Acc>(wr) * static_cast<Acc>(load_f32(x + r * x_stride + idx % width)));
+}
+
 // ---- per-head unit norm, weight and gate -------------------------------------------------------
 // out[t, h, :] = o[t, h, :] / sqrt(mean_j o[t, h, j]^2 + eps) * w[h, :] * silu(g[t, h, :]); w may be
 // absent. One wavefront per (token, head). o is float (what a recurrence or attention left); g and
-// out have the activation type.
+// out have the activation type. `sigmoid_gate`: the gate is sigmoid(g) instead of silu(g). `extra`: a head of o holds so
+// many more channels behind its dv; with `floor` [tokens, heads] the first of them is a normaliser: the head's dv values
+// are divided by max(|it|, floor[t, h]) + 1e-6 before the norm.
 template <typename T, typename Acc>
 __global__ void __launch_bounds__(256) headnorm_gate_kernel(T* __restrict__ out, int64_t out_stride, const float* __restrict__ o,
                                                             const T* __restrict__ g, int64_t g_stride, const float* __restrict__ w,
-                                                            int tokens, int heads, int dv, float eps, float out_scale, int parts, int64_t part_stride) {
+                                                            int tokens, int heads, int dv, float eps, float out_scale, int parts, int64_t part_stride,
+                                                            int sigmoid_gate, int extra, const float* __restrict__ floor) {
   const int64_t unit = static_cast<int64_t>(blockIdx.x) * 4 + threadIdx.x / kWave;
   if (unit >= static_cast<int64_t>(tokens) * heads) return;
   const int lane = threadIdx.x % kWave;
   const int t = static_cast<int>(unit / heads), h = static_cast<int>(unit % heads);
-  const float* src = o + (static_cast<int64_t>(t) * heads + h) * dv;
+  const float* src = o + (static_cast<int64_t>(t) * heads + h) * (dv + extra);
+  float under = 1.f;      // what the head's values are divided by first
+  if (floor) {
+    float n = 0.f;
+    for (int p = 0; p < parts; ++p) n += src[p * part_stride + dv];
+    under = fmaxf(fabsf(n), floor[static_cast<int64_t>(t) * heads + h]) + 1e-6f;
+  }
   // (o may come in parts, left by blocks that each held a share of the key channels: they are added here, in their order)
   constexpr int kOwn = 4;      // values a lane keeps between the sum of squares and the scaling (heads up to 256 wide; wider ones are added again)
   float own[kOwn];
@@ -62,12 +107,14 @@ __global__ void __launch_bounds__(256) headnorm_gate_kernel(T* __restrict__ out,
     float v = 0.f;
     if (j < dv)
       for (int p = 0; p < parts; ++p) v += src[p * part_stride + j];
+    if (floor) v /= under;
     own[c] = v;
     ss += static_cast<Acc>(v) * static_cast<Acc>(v);
   }
   for (int j = lane + kOwn * kWave; j < dv; j += kWave) {
     float v = 0.f;
     for (int p = 0; p < parts; ++p) v += src[p * part_stride + j];
+    if (floor) v /= under;
     ss += static_cast<Acc>(v) * static_cast<Acc>(v);
   }
   ss = wave_sum(ss);
@@ -76,7 +123,7 @@ __global__ void __launch_bounds__(256) headnorm_gate_kernel(T* __restrict__ out,
   T* dst = out + static_cast<int64_t>(t) * out_stride + static_cast<int64_t>(h) * dv;
   for (int j = lane; j < dv; j += kWave) {
     const Acc z = static_cast<Acc>(load_f32(gate + j));
-    const Acc silu = z / (static_cast<Acc>(1) + exp(-z));
+    const Acc silu = (sigmoid_gate ? static_cast<Acc>(1) : z) / (static_cast<Acc>(1) + exp(-z));
     float v = 0.f;
     if (j < kOwn * kWave) {
 #pragma unroll
@@ -84,6 +131,7 @@ __global__ void __launch_bounds__(256) headnorm_gate_kernel(T* __restrict__ out,
         if (j == lane + c * kWave) v = own[c];
     } else {
       for (int p = 0; p < parts; ++p) v += src[p * part_stride + j];
+      if (floor) v /= under;
     }
     Acc y = static_cast<Acc>(v) * inv;
     if (w) y *= static_cast<Acc>(w[h * dv + j]);
@@ -93,7 +141,7 @@ __global__ void __launch_bounds__(256) headnorm_gate_kernel(T* __restrict__ out,
 
 // ---- activations -------------------------------------------------------------------------------
 // kind 0: xIELU with a = softplus(p) and b = 1/2 + softplus(q) given: z > 0: a z^2 + z/2; else b (exp(z) - 1 - z) + z/2.
-// kind 1: tanh. In place or not; rows of `width` values with a row stride.
+// kind 1: tanh. kind 2: silu, z sigmoid(z). In place or not; rows of `width` values with a row stride.
 template <typename T, typename Acc>
 __global__ void __launch_bounds__(256) activation_kernel(T* __restrict__ out, int64_t out_stride, const T* __restrict__ x, int64_t x_stride,
                                                          int64_t rows, int width, int kind, float a, float b) {
@@ -105,8 +153,10 @@ __global__ void __launch_bounds__(256) activation_kernel(T* __restrict__ out, in
   Acc y;
   if (kind == 0) {
     y = z > 0 ? static_cast<Acc>(a) * z * z + z / 2 : static_cast<Acc>(b) * (expm1(z) - z) + z / 2;
-  } else {
+  } else if (kind == 1) {
     y = tanh(z);
+  } else {
+    y = z / (static_cast<Acc>(1) + exp(-z));
   }
   store_f32(out + r * out_stride + c, static_cast<float>(y));
 }
@@ -161,21 +211,41 @@ extern "C" int alofa_layernorm(void* out, int out_dtype, const float* x, const f
   return check_launch("layernorm");
 }
 
+extern "C" int alofa_layernorm_add(float* residual, const float* x, const float* w, const float* b, int n_rows, int width, float eps, int exact, hipStream_t stream) {
+  ALOFA_REQUIRE(n_rows >= 0 && width > 0 && eps > 0.f, "layernorm_add: bad sizes (rows=%d width=%d)", n_rows, width);
+  if (n_rows == 0) return 0;
+  if (exact) layernorm_add_kernel<double><<<n_rows, 256, 0, stream>>>(residual, x, w, b, width, eps);
+  else layernorm_add_kernel<float><<<n_rows, 256, 0, stream>>>(residual, x, w, b, width, eps);
+  return check_launch("layernorm_add");
+}
+
+extern "C" int alofa_add_row_scaled(float* out, const void* x, int64_t x_stride, int dtype, const float* w, int64_t rows, int width, int exact, hipStream_t stream) {
+  ALOFA_REQUIRE(rows >= 0 && width > 0, "add_row_scaled: bad sizes");
+  if (rows == 0) return 0;
+  const unsigned grid = static_cast<unsigned>((rows * width + 255) / 256);
+  if (exact && dtype == kF32) add_row_scaled_kernel<float, double><<<grid, 256, 0, stream>>>(out, static_cast<const float*>(x), x_stride, w, rows, width);
+  else if (dtype == kF32) add_row_scaled_kernel<float, float><<<grid, 256, 0, stream>>>(out, static_cast<const float*>(x), x_stride, w, rows, width);
+  else add_row_scaled_kernel<bf16_t, float><<<grid, 256, 0, stream>>>(out, static_cast<const bf16_t*>(x), x_stride, w, rows, width);
+  return check_launch("add_row_scaled");
+}
+
 extern "C" int alofa_headnorm_gate(void* out, int64_t out_stride, const float* o, const void* g, int64_t g_stride, int dtype, const float* w,
-                                   int tokens, int heads, int dv, float eps, float out_scale, int parts, int64_t part_stride, int exact, hipStream_t stream) {
+                                   int tokens, int heads, int dv, float eps, float out_scale, int parts, int64_t part_stride, int exact,
+                                   int sigmoid_gate, int extra, const float* floor, hipStream_t stream) {
+  ALOFA_REQUIRE(extra >= 0 && (!floor || extra >= 1), "headnorm_gate: a normaliser needs a channel behind the head's own");
   ALOFA_REQUIRE(tokens >= 0 && heads > 0 && dv > 0 && eps > 0.f && parts >= 1, "headnorm_gate: bad sizes (tokens=%d heads=%d dv=%d)", tokens, heads, dv);
   ALOFA_REQUIRE(!exact || dtype == kF32, "headnorm_gate: the exact path is float32");
   if (tokens == 0) return 0;
   const unsigned grid = static_cast<unsigned>((static_cast<int64_t>(tokens) * heads + 3) / 4);
-  if (exact) headnorm_gate_kernel<float, double><<<grid, 256, 0, stream>>>(static_cast<float*>(out), out_stride, o, static_cast<const float*>(g), g_stride, w, tokens, heads, dv, eps, out_scale, parts, part_stride);
-  else if (dtype == kF32) headnorm_gate_kernel<float, float><<<grid, 256, 0, stream>>>(static_cast<float*>(out), out_stride, o, static_cast<const float*>(g), g_stride, w, tokens, heads, dv, eps, out_scale, parts, part_stride);
-  else headnorm_gate_kernel<bf16_t, float><<<grid, 256, 0, stream>>>(static_cast<bf16_t*>(out), out_stride, o, static_cast<const bf16_t*>(g), g_stride, w, tokens, heads, dv, eps, out_scale, parts, part_stride);
+  if (exact) headnorm_gate_kernel<float, double><<<grid, 256, 0, stream>>>(static_cast<float*>(out), out_stride, o, static_cast<const float*>(g), g_stride, w, tokens, heads, dv, eps, out_scale, parts, part_stride, sigmoid_gate, extra, floor);
+  else if (dtype == kF32) headnorm_gate_kernel<float, float><<<grid, 256, 0, stream>>>(static_cast<float*>(out), out_stride, o, static_cast<const float*>(g), g_stride, w, tokens, heads, dv, eps, out_scale, parts, part_stride, sigmoid_gate, extra, floor);
+  else headnorm_gate_kernel<bf16_t, float><<<grid, 256, 0, stream>>>(static_cast<bf16_t*>(out), out_stride, o, static_cast<const bf16_t*>(g), g_stride, w, tokens, heads, dv, eps, out_scale, parts, part_stride, sigmoid_gate, extra, floor);
   return check_launch("headnorm_gate");
 }
 
 extern "C" int alofa_activation(void* out, int64_t out_stride, const void* x, int64_t x_stride, int dtype, int64_t rows, int width,
                                 int kind, float a, float b, int exact, hipStream_t stream) {
-  ALOFA_REQUIRE(rows >= 0 && width > 0 && (kind == 0 || kind == 1), "activation: bad arguments (rows=%lld width=%d kind=%d)", (long long)rows, width, kind);
+  ALOFA_REQUIRE(rows >= 0 && width > 0 && kind >= 0 && kind <= 2, "activation: bad arguments (rows=%lld width=%d kind=%d)", (long long)rows, width, kind);
   ALOFA_REQUIRE(!exact || dtype == kF32, "activation: the exact path is float32");
   if (rows == 0) return 0;
   const unsigned grid = blocks_of(rows * width);

@@ -407,11 +407,78 @@ __global__ void __launch_bounds__((KL <= 8 || KL == 64) ? 512 : 256) linear_recu
   }
 }
 
+// ---- exponential gates kept in range by a running maximum (the matrix memory of xLSTM) ---------------------------
+// Per request and head, over the request's rows in order, with m the running maximum kept in the request's slot (0 for a new request):
+//   i = cap tanh(zi / cap), f = log sigmoid(cap tanh(zf / cap));  m' = max(f + m, i);  keep = exp(f + m - m'), take = exp(i - m')
+// gates[0 / 1 / 2][t, head] = keep / take / exp(-m') (three planes of [rows, heads]). One thread per (request, head): the scan is a handful of operations a row.
+__global__ void __launch_bounds__(64) gate_scan_kernel(float* __restrict__ gates, const float* __restrict__ z, int64_t z_stride, float* __restrict__ state,
+                                                       const int32_t* __restrict__ req_slot, const int32_t* __restrict__ row_off, int requests, int64_t rows, int heads, float cap) {
+  const int idx = blockIdx.x * 64 + threadIdx.x;
+  if (idx >= requests * heads) return;
+  const int r = idx / heads, h = idx % heads;
+  const int row0 = row_off ? row_off[r] : r, end = row_off ? row_off[r + 1] : r + 1;
+  float* kept = state + static_cast<int64_t>(req_slot[r]) * heads + h;
+  float m = *kept;
+  for (int t = row0; t < end; ++t) {
+    const float zi = z[t * z_stride + h], zf = z[t * z_stride + heads + h];
+    const float gi = cap * tanhf(zi / cap), x = cap * tanhf(zf / cap);
+    const float gf = -(fmaxf(-x, 0.f) + log1pf(expf(-fabsf(x))));      // log sigmoid(x)
+    const float next = fmaxf(gf + m, gi);
+    float* g = gates + static_cast<int64_t>(t) * heads + h;
+    g[0] = expf(gf + m - next);
+    g[rows * heads] = expf(gi - next);
+    g[2 * rows * heads] = expf(-next);
+    m = next;
+  }
+  *kept = m;
+}
+
+// The operands of the recurrence as float rows, gates applied: qf = q, kf = take * k, decay[t, head, :] = keep, vf = [v, 1] per head
+// (the channel of ones carries the normaliser n_t = keep n + take k through the same recurrence: its read-out is n . q).
+template <typename T>
+__global__ void __launch_bounds__(256) gated_operands_kernel(float* __restrict__ qf, float* __restrict__ kf, float* __restrict__ vf, float* __restrict__ decay,
+                                                             const T* __restrict__ q, int64_t q_stride, const T* __restrict__ k, int64_t k_stride,
+                                                             const T* __restrict__ v, int64_t v_stride, const float* __restrict__ gates,
+                                                             int64_t rows, int heads, int dk, int dv) {
+  const int per_row = heads * (dk + dv + 1);
+  const int64_t idx = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+  if (idx >= rows * per_row) return;
+  const int64_t t = idx / per_row;
+  const int e = static_cast<int>(idx % per_row);
+  if (e < heads * dk) {
+    const float* g = gates + t * heads + e / dk;
+    qf[t * heads * dk + e] = load_f32(q + t * q_stride + e);
+    kf[t * heads * dk + e] = g[rows * heads] * load_f32(k + t * k_stride + e);
+    decay[t * heads * dk + e] = g[0];
+  } else {
+    const int c = e - heads * dk, h = c / (dv + 1), j = c % (dv + 1);
+    vf[t * heads * (dv + 1) + c] = j < dv ? load_f32(v + t * v_stride + h * dv + j) : 1.f;
+  }
+}
+
 }  // namespace alofa
 
 using namespace alofa;
 
 static inline unsigned blocks_of(int64_t n) { return static_cast<unsigned>((n + 255) / 256); }
+
+extern "C" int alofa_gate_scan(float* gates, const float* z, int64_t z_stride, float* state, const int32_t* req_slot, const int32_t* row_off, int requests,
+                               int64_t rows, int heads, float cap, hipStream_t stream) {
+  ALOFA_REQUIRE(requests >= 0 && heads > 0 && cap > 0.f, "gate_scan: bad arguments (requests=%d heads=%d cap=%g)", requests, heads, cap);
+  if (requests == 0) return 0;
+  gate_scan_kernel<<<(requests * heads + 63) / 64, 64, 0, stream>>>(gates, z, z_stride, state, req_slot, row_off, requests, rows, heads, cap);
+  return check_launch("gate_scan");
+}
+
+extern "C" int alofa_gated_operands(float* qf, float* kf, float* vf, float* decay, const void* q, int64_t q_stride, const void* k, int64_t k_stride,
+                                    const void* v, int64_t v_stride, int dtype, const float* gates, int64_t rows, int heads, int dk, int dv, hipStream_t stream) {
+  ALOFA_REQUIRE(rows >= 0 && heads > 0 && dk > 0 && dv > 0, "gated_operands: bad sizes");
+  if (rows == 0) return 0;
+  const unsigned grid = blocks_of(rows * heads * (dk + dv + 1));
+  if (dtype == kF32) gated_operands_kernel<float><<<grid, 256, 0, stream>>>(qf, kf, vf, decay, static_cast<const float*>(q), q_stride, static_cast<const float*>(k), k_stride, static_cast<const float*>(v), v_stride, gates, rows, heads, dk, dv);
+  else gated_operands_kernel<bf16_t><<<grid, 256, 0, stream>>>(qf, kf, vf, decay, static_cast<const bf16_t*>(q), q_stride, static_cast<const bf16_t*>(k), k_stride, static_cast<const bf16_t*>(v), v_stride, gates, rows, heads, dk, dv);
+  return check_launch("gated_operands");
+}
 
 extern "C" int alofa_short_conv(void* out, int out_dtype, const void* h, int h_dtype, const float* w, const void* state, const int32_t* req_slot,
                                 const int32_t* row_off, const int32_t* req_of_row, int rows, int width, int taps, int exact, hipStream_t stream) {

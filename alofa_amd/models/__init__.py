@@ -2,10 +2,12 @@
 from ..config.registry import register_architecture
 from .qwen2 import Qwen2Config
 from .rerupel import RerupelConfig
+from .retotar import RetotarConfig
 from .tugalix import TugalixConfig
 
 register_architecture(Qwen2Config.architecture, Qwen2Config)
 register_architecture(TugalixConfig.architecture, TugalixConfig)
 register_architecture(RerupelConfig.architecture, RerupelConfig)
+register_architecture(RetotarConfig.architecture, RetotarConfig)
 
-__all__ = ["Qwen2Config", "RerupelConfig", "TugalixConfig"]
+__all__ = ["Qwen2Config", "RerupelConfig", "RetotarConfig", "TugalixConfig"]

@@ -804,6 +804,73 @@ _argmax_scratch: dict = {}
 _argmax_retired: list = []       # outgrown scratch buffers: a captured step may still address them
 
 
+def turn_norm_write(qkv: torch.Tensor, positions: torch.Tensor, qk_table: tuple, v_table: Optional[tuple], heads: int, kv_heads: int, d: int, dv: int,
+                    eps: float, unit_norm: bool, exact: bool, slots: Optional[torch.Tensor] = None, k_cache: Optional[torch.Tensor] = None,
+                    v_cache: Optional[torch.Tensor] = None) -> None:
+    """What a step's projections become before attention with turned values. ``qkv`` [T, heads * d + kv_heads * (d + dv)]: query heads, key
+    heads, value heads side by side (``kv_heads`` 0: queries only). Queries and keys are turned on their first channels by ``qk_table``
+    (cos, sin float32 [n, pairs]: channel i with i + pairs) and, with ``unit_norm``, divided by their root mean square over d; values are
+    turned on all channels by ``v_table`` [n, dv / 2]. Queries are left in place; keys go to ``k_cache`` [pages, kv_heads, page, d] and
+    values to ``v_cache`` [pages, kv_heads, page, dv] at ``slots`` int64 [T]."""
+    _gpu("qkv", qkv, None, 2), _gpu("positions", positions, torch.int32, 1), _contig("positions", positions)
+    T = qkv.shape[0]
+    cos, sin = qk_table
+    _gpu("cos", cos, torch.float32, 2), _gpu("sin", sin, torch.float32, 2), _contig("cos", cos), _contig("sin", sin)
+    half = cos.shape[1]
+    if qkv.shape[1] != heads * d + kv_heads * (d + dv) or positions.shape[0] != T or cos.shape != sin.shape or 2 * half > d:
+        raise AlofaError("shape_mismatch", "rows, positions or tables do not fit", f"qkv={tuple(qkv.shape)} heads={heads} kv_heads={kv_heads} d={d} dv={dv} table={tuple(cos.shape)}")
+    cv = sv = None
+    block = 0
+    if kv_heads:
+        cv, sv = v_table
+        _gpu("cos_v", cv, torch.float32, 2), _gpu("sin_v", sv, torch.float32, 2), _contig("cos_v", cv), _contig("sin_v", sv)
+        _gpu("slots", slots, torch.int64, 1), _contig("slots", slots), _gpu("k_cache", k_cache, qkv.dtype, 4), _gpu("v_cache", v_cache, qkv.dtype, 4)
+        _contig("k_cache", k_cache), _contig("v_cache", v_cache)
+        block = k_cache.shape[2]
+        if (cv.shape[1] != dv // 2 or cv.shape != sv.shape or cv.shape[0] < cos.shape[0] or slots.shape[0] != T or tuple(k_cache.shape[1:]) != (kv_heads, block, d)
+                or tuple(v_cache.shape) != (k_cache.shape[0], kv_heads, block, dv)):
+            raise AlofaError("shape_mismatch", "caches, slots or the values' table do not fit", f"k={tuple(k_cache.shape)} v={tuple(v_cache.shape)} table={tuple(cv.shape)} slots={tuple(slots.shape)}")
+    _call("alofa_turn_norm_write", _ptr(qkv), _L(_rows("qkv", qkv)), _I(dtype_code(qkv)), _ptr(positions), _ptr(cos), _ptr(sin), _I(half), _ptr(cv), _ptr(sv),
+          _ptr(slots), _ptr(k_cache), _ptr(v_cache), _I(block), _I(T), _I(heads), _I(kv_heads), _I(d), _I(dv), _F(eps), _I(int(unit_norm)), _I(int(exact)), _stream())
+
+
+def talking_attention(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_table: torch.Tensor,
+                      req_of_token: Optional[torch.Tensor], positions: torch.Tensor, heads: int, kv_heads: int, d: int, dv: int, window: Optional[int],
+                      scale: float, talk: Optional[torch.Tensor], v_table: Optional[tuple], gate: Optional[torch.Tensor], exact: bool = False) -> None:
+    """out[t, h] = turn_back(sum_j (sum_g talk[h, g] softmax_g(t, j)) v[j, h // group]) * sigmoid(gate[t, h]): softmax per query head g over
+    the keys row t may see (its request's, up to its position; the last ``window`` of them), weights mixed over heads by ``talk`` [heads,
+    heads] (None: not mixed), values [pages, kv_heads, page, dv] that were turned by their positions (``v_table``: the result is turned back
+    by the row's; None: nothing is turned). ``q`` [T, heads * d] and ``out``, ``gate`` [T, heads * dv] rows (row strides allowed)."""
+    _gpu("out", out, None, 2), _gpu("q", q, out.dtype, 2), _gpu("k_cache", k_cache, out.dtype, 4), _gpu("v_cache", v_cache, out.dtype, 4)
+    _contig("k_cache", k_cache), _contig("v_cache", v_cache), _gpu("block_table", block_table, torch.int32, 2), _contig("block_table", block_table)
+    _gpu("positions", positions, torch.int32, 1), _contig("positions", positions)
+    T, block = q.shape[0], k_cache.shape[2]
+    if (tuple(q.shape) != (T, heads * d) or tuple(out.shape) != (T, heads * dv) or tuple(k_cache.shape[1:]) != (kv_heads, block, d)
+            or tuple(v_cache.shape) != (k_cache.shape[0], kv_heads, block, dv) or positions.shape[0] != T):
+        raise AlofaError("shape_mismatch", "attention operands do not fit", f"out={tuple(out.shape)} q={tuple(q.shape)} k={tuple(k_cache.shape)} v={tuple(v_cache.shape)} heads={heads} kv_heads={kv_heads} d={d} dv={dv}")
+    if req_of_token is not None:
+        _gpu("req_of_token", req_of_token, torch.int32, 1), _contig("req_of_token", req_of_token)
+    elif block_table.shape[0] < T:
+        raise AlofaError("shape_mismatch", "without a request per row every row is a request of its own", f"rows={T} tables={block_table.shape[0]}")
+    if talk is not None:
+        _gpu("talk", talk, torch.float32, 2), _contig("talk", talk)
+        if tuple(talk.shape) != (heads, heads):
+            raise AlofaError("shape_mismatch", "the heads' mixing matrix is [heads, heads]", f"talk={tuple(talk.shape)}")
+    cv = sv = None
+    if v_table is not None:
+        cv, sv = v_table
+        _gpu("cos_v", cv, torch.float32, 2), _gpu("sin_v", sv, torch.float32, 2), _contig("cos_v", cv), _contig("sin_v", sv)
+        if cv.shape[1] != dv // 2 or cv.shape != sv.shape:
+            raise AlofaError("shape_mismatch", "the values' table does not fit", f"table={tuple(cv.shape)} dv={dv}")
+    if gate is not None:
+        _gpu("gate", gate, out.dtype, 2)
+        if gate.shape != out.shape:
+            raise AlofaError("shape_mismatch", "one gate per output", f"gate={tuple(gate.shape)} out={tuple(out.shape)}")
+    _call("alofa_talking_attention", _ptr(out), _L(_rows("out", out)), _ptr(q), _L(_rows("q", q)), _ptr(k_cache), _ptr(v_cache), _I(dtype_code(out)),
+          _ptr(block_table), _I(block_table.shape[1]), _ptr(req_of_token), _ptr(positions), _I(T), _I(heads), _I(kv_heads), _I(d), _I(dv), _I(block),
+          _I(int(window or 0)), _F(scale), _ptr(talk), _ptr(cv), _ptr(sv), _ptr(gate), _L(_rows("gate", gate) if gate is not None else 0), _I(int(exact)), _stream())
+
+
 def _store_operands(store, store_index, n: int):
     if (store is None) != (store_index is None):
         raise AlofaError("invalid_argument", "a token store goes with the index of every row's place in it")
@@ -912,13 +979,40 @@ def layernorm(out: torch.Tensor, x: torch.Tensor, w: torch.Tensor, b: torch.Tens
           _I(int(exact)), _stream())
 
 
+def layernorm_add(residual: torch.Tensor, x: torch.Tensor, w: torch.Tensor, b: torch.Tensor, eps: float, exact: bool = False) -> None:
+    """residual[r] += (x[r] - mean) / sqrt(var + eps) * w + b: the norm behind a sub-layer on its way into the stream (all float32)."""
+    _gpu("residual", residual, torch.float32, 2), _gpu("x", x, torch.float32, 2), _gpu("w", w, torch.float32, 1), _gpu("b", b, torch.float32, 1)
+    _contig("residual", residual), _contig("x", x), _contig("w", w), _contig("b", b)
+    n, h = residual.shape
+    if tuple(x.shape) != (n, h) or w.shape[0] != h or b.shape[0] != h:
+        raise AlofaError("shape_mismatch", "norm width does not fit", f"residual={tuple(residual.shape)} x={tuple(x.shape)} w={tuple(w.shape)} b={tuple(b.shape)}")
+    _call("alofa_layernorm_add", _ptr(residual), _ptr(x), _ptr(w), _ptr(b), _I(n), _I(h), _F(eps), _I(int(exact)), _stream())
+
+
+def add_row_scaled(out: torch.Tensor, x: torch.Tensor, w: torch.Tensor, exact: bool = False) -> None:
+    """out[t] += w[t] * x[t]: ``out`` float32 [T, h] contiguous, ``x`` [T, h] rows of any type (row strides allowed), ``w`` float32 [T]."""
+    _gpu("out", out, torch.float32, 2), _gpu("x", x, None, 2), _gpu("w", w, torch.float32, 1), _contig("out", out), _contig("w", w)
+    if x.shape != out.shape or w.shape[0] != out.shape[0]:
+        raise AlofaError("shape_mismatch", "one weight per row; rows of one shape", f"out={tuple(out.shape)} x={tuple(x.shape)} w={tuple(w.shape)}")
+    _call("alofa_add_row_scaled", _ptr(out), _ptr(x), _L(_rows("x", x)), _I(dtype_code(x)), _ptr(w), _L(out.shape[0]), _I(out.shape[1]), _I(int(exact)), _stream())
+
+
 def headnorm_gate(out: torch.Tensor, o: torch.Tensor, gate: torch.Tensor, weight: Optional[torch.Tensor], heads: int, dv: int,
-                  eps: float, exact: bool, out_scale: float = 1.0, parts: int = 1) -> None:
+                  eps: float, exact: bool, out_scale: float = 1.0, parts: int = 1, gate_kind: str = "silu", extra: int = 0,
+                  floor: Optional[torch.Tensor] = None) -> None:
     """out[t, h, :] = o[t, h, :] / sqrt(mean(o[t, h, :]^2) + eps) * weight[h, :] * silu(gate[t, h, :]); ``o`` float32
     [T, heads * dv] contiguous, or [P, T, heads * dv] whose first ``parts`` are added first (read-outs that
     ``linear_recurrence`` left in parts); ``gate`` and ``out`` rows of heads * dv in the activation dtype (row strides
-    allowed), ``weight`` float32 [heads * dv] or None."""
+    allowed), ``weight`` float32 [heads * dv] or None. ``gate_kind`` "sigmoid": the gate is sigmoid(gate) instead. ``extra``: a head
+    of ``o`` holds so many channels more than its dv (o is [.., T, heads * (dv + extra)]); with ``floor`` float32 [T, heads] the first of
+    them is a normaliser: the head's values are divided by max(|it|, floor) + 1e-6 before the norm."""
     _gpu("out", out, None, 2), _gpu("o", o, torch.float32), _gpu("gate", gate, out.dtype, 2), _contig("o", o)
+    if gate_kind not in ("silu", "sigmoid") or extra < 0 or (floor is not None and extra < 1):
+        raise AlofaError("invalid_argument", "the gate is silu or sigmoid; a normaliser needs a channel of its own", f"gate_kind={gate_kind} extra={extra}")
+    if floor is not None:
+        _gpu("floor", floor, torch.float32, 2), _contig("floor", floor)
+        if tuple(floor.shape) != (o.shape[-2], heads):
+            raise AlofaError("shape_mismatch", "one floor per row and head", f"floor={tuple(floor.shape)}")
     part_stride = 0
     if o.dim() == 3:
         if not 1 <= parts <= o.shape[0]:
@@ -927,7 +1021,7 @@ def headnorm_gate(out: torch.Tensor, o: torch.Tensor, gate: torch.Tensor, weight
     elif o.dim() != 2 or parts != 1:
         raise AlofaError("shape_mismatch", "read-outs are [T, heads * dv] or parts of that", f"o={tuple(o.shape)} parts={parts}")
     T = o.shape[0]
-    if o.shape[1] != heads * dv or tuple(out.shape) != (T, heads * dv) or tuple(gate.shape) != (T, heads * dv):
+    if o.shape[1] != heads * (dv + extra) or tuple(out.shape) != (T, heads * dv) or tuple(gate.shape) != (T, heads * dv):
         raise AlofaError("shape_mismatch", "head norm operands do not fit", f"out={tuple(out.shape)} o={tuple(o.shape)} gate={tuple(gate.shape)} heads={heads} dv={dv}")
     if weight is not None:
         _gpu("weight", weight, torch.float32, 1), _contig("weight", weight)
@@ -936,17 +1030,18 @@ def headnorm_gate(out: torch.Tensor, o: torch.Tensor, gate: torch.Tensor, weight
     if exact and out.dtype is not torch.float32:
         raise AlofaError("invalid_argument", "the exact path is float32 throughout", f"out={out.dtype}")
     _call("alofa_headnorm_gate", _ptr(out), _L(_rows("out", out)), _ptr(o), _ptr(gate), _L(_rows("gate", gate)), _I(dtype_code(out)), _ptr(weight),
-          _I(T), _I(heads), _I(dv), _F(eps), _F(out_scale), _I(parts), _L(part_stride), _I(int(exact)), _stream())
+          _I(T), _I(heads), _I(dv), _F(eps), _F(out_scale), _I(parts), _L(part_stride), _I(int(exact)),
+          _I(int(gate_kind == "sigmoid")), _I(extra), _ptr(floor), _stream())
 
 
-XIELU, TANH = 0, 1
+XIELU, TANH, SILU = 0, 1, 2
 
 
 def activation(out: torch.Tensor, x: torch.Tensor, kind: int, a: float = 0.0, b: float = 0.0, exact: bool = False) -> None:
     """out = act(x) element by element on rows ([T, n], row strides allowed; out may be x). ``XIELU`` with a = softplus(p),
-    b = 1/2 + softplus(q): z > 0: a z^2 + z/2, else b (exp(z) - 1 - z) + z/2. ``TANH``."""
+    b = 1/2 + softplus(q): z > 0: a z^2 + z/2, else b (exp(z) - 1 - z) + z/2. ``TANH``. ``SILU``: z sigmoid(z)."""
     _gpu("out", out, None, 2), _gpu("x", x, out.dtype, 2)
-    if out.shape != x.shape or kind not in (XIELU, TANH):
+    if out.shape != x.shape or kind not in (XIELU, TANH, SILU):
         raise AlofaError("shape_mismatch", "activation operands do not fit", f"out={tuple(out.shape)} x={tuple(x.shape)} kind={kind}")
     if exact and out.dtype is not torch.float32:
         raise AlofaError("invalid_argument", "the exact path is float32 throughout", f"out={out.dtype}")
@@ -1126,6 +1221,34 @@ def linear_recurrence(out: torch.Tensor, q: torch.Tensor, k: torch.Tensor, v: to
     return used.value
 
 
+def gate_scan(gates: torch.Tensor, z: torch.Tensor, state: torch.Tensor, rows: RowsOfRequests, heads: int, cap: float) -> None:
+    """Exponential gates kept in range by a running maximum m (``state`` float32 [slots, heads], read and left there), per request over
+    its rows in order: with z [T, 2 * heads] float32 (input gates' then forget gates' products), i = cap tanh(zi / cap),
+    f = log sigmoid(cap tanh(zf / cap)), m' = max(f + m, i): gates[0], [1], [2] = exp(f + m - m'), exp(i - m'), exp(-m'), each float32 [T, heads] (``gates`` [3, T, heads])."""
+    _gpu("gates", gates, torch.float32, 3), _contig("gates", gates), _gpu("z", z, torch.float32, 2), _gpu("state", state, torch.float32, 2), _contig("state", state)
+    T = z.shape[0]
+    if tuple(gates.shape) != (3, T, heads) or z.shape[1] != 2 * heads or state.shape[1] != heads or T != rows.rows or not cap > 0:
+        raise AlofaError("shape_mismatch", "gate operands do not fit", f"gates={tuple(gates.shape)} z={tuple(z.shape)} state={tuple(state.shape)} heads={heads} rows={rows.rows}")
+    rows.fits("state", state)
+    _call("alofa_gate_scan", _ptr(gates), _ptr(z), _L(_rows("z", z)), _ptr(state), _ptr(rows.slots), _ptr(rows.offsets), _I(rows.requests), _L(T), _I(heads), _F(cap), _stream())
+
+
+def gated_operands(qf: torch.Tensor, kf: torch.Tensor, vf: torch.Tensor, decay: torch.Tensor, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
+                   gates: torch.Tensor, heads: int, dk: int, dv: int) -> None:
+    """What ``linear_recurrence`` takes for a memory with gates per row and head (``gate_scan``), as float32 rows: qf = q, kf = take * k,
+    decay = keep for every key channel of the head, vf [T, heads * (dv + 1)] = the head's values and a one (whose read-out is the normaliser)."""
+    T = q.shape[0]
+    for n, t, w in (("qf", qf, heads * dk), ("kf", kf, heads * dk), ("decay", decay, heads * dk), ("vf", vf, heads * (dv + 1))):
+        _gpu(n, t, torch.float32, 2), _contig(n, t)
+        if tuple(t.shape) != (T, w):
+            raise AlofaError("shape_mismatch", "the float operands do not fit", f"operand={n} shape={tuple(t.shape)} rows={T} width={w}")
+    _gpu("q", q, None, 2), _gpu("k", k, q.dtype, 2), _gpu("v", v, q.dtype, 2), _gpu("gates", gates, torch.float32, 3), _contig("gates", gates)
+    if tuple(q.shape) != (T, heads * dk) or tuple(k.shape) != (T, heads * dk) or tuple(v.shape) != (T, heads * dv) or tuple(gates.shape) != (3, T, heads):
+        raise AlofaError("shape_mismatch", "the rows do not fit", f"q={tuple(q.shape)} k={tuple(k.shape)} v={tuple(v.shape)} gates={tuple(gates.shape)}")
+    _call("alofa_gated_operands", _ptr(qf), _ptr(kf), _ptr(vf), _ptr(decay), _ptr(q), _L(_rows("q", q)), _ptr(k), _L(_rows("k", k)), _ptr(v), _L(_rows("v", v)),
+          _I(dtype_code(q)), _ptr(gates), _L(T), _I(heads), _I(dk), _I(dv), _stream())
+
+
 # ------------------------------------------------------------- scaled sub-layers, pair embedding, stream joins, choices among experts
 
 def pair_embed(out: torch.Tensor, table: torch.Tensor, ids: torch.Tensor, scale: float = 1.0, store: Optional[torch.Tensor] = None,
@@ -1222,9 +1345,31 @@ def route_top(z: torch.Tensor, dense: torch.Tensor, chosen: torch.Tensor, weight
     _call("alofa_route_top", _ptr(z), _ptr(dense), _ptr(chosen), _ptr(weights), _I(T), _I(E), _I(top), _F(scale), _I(int(renormalize)), _I(int(exact)), _stream())
 
 
+def route_groups(z: torch.Tensor, correction: Optional[torch.Tensor], dense: torch.Tensor, chosen: torch.Tensor, weights: torch.Tensor,
+                 pass_weight: torch.Tensor, top: int, passing: int = 0, groups: int = 1, keep: int = 1, scale: float = 1.0, renormalize: bool = False,
+                 exact: bool = False) -> None:
+    """The choice by softmax scores: s = softmax(z) over all E columns of z [T, E]; the choice goes by s + correction; the experts form
+    ``groups`` equal groups of neighbours, of which the ``keep`` with the largest member stay in the choice; the ``top`` largest of those are
+    taken (``chosen`` int32 [T, top]), weighted by their s (``weights``). The last ``passing`` experts have no matrices: ``dense`` float32
+    [T, E - passing] holds the weights of the others, ``pass_weight`` float32 [T] the summed weights of taken experts without matrices."""
+    _gpu("z", z, torch.float32, 2), _gpu("dense", dense, torch.float32, 2), _gpu("chosen", chosen, torch.int32, 2), _gpu("weights", weights, torch.float32, 2)
+    _gpu("pass_weight", pass_weight, torch.float32, 1)
+    for n, t in (("z", z), ("dense", dense), ("chosen", chosen), ("weights", weights), ("pass_weight", pass_weight)):
+        _contig(n, t)
+    T, E = z.shape
+    if correction is not None:
+        _gpu("correction", correction, torch.float32, 1), _contig("correction", correction)
+    if (tuple(dense.shape) != (T, E - passing) or tuple(chosen.shape) != (T, top) or tuple(weights.shape) != (T, top) or pass_weight.shape[0] != T
+            or not 0 < top <= E <= MAX_EXPERTS or not 0 <= passing < E or (correction is not None and correction.shape[0] != E)
+            or groups < 1 or E % groups or not 1 <= keep <= groups or top > keep * (E // groups)):
+        raise AlofaError("shape_mismatch", "the choice's operands do not fit", f"z={tuple(z.shape)} dense={tuple(dense.shape)} chosen={tuple(chosen.shape)} top={top} passing={passing} groups={groups} keep={keep}")
+    _call("alofa_route_groups", _ptr(z), _ptr(correction), _ptr(dense), _ptr(chosen), _ptr(weights), _ptr(pass_weight), _I(T), _I(E), _I(passing), _I(top),
+          _I(groups), _I(keep), _F(scale), _I(int(renormalize)), _I(int(exact)), _stream())
+
+
 def clamped_glu(act: torch.Tensor, g: torch.Tensor, u: torch.Tensor, dense: Optional[torch.Tensor], experts: int, ff: int, shared_ff: int,
-                limit: float, shared_limit: float, slope: float, exact: bool = False) -> None:
-    """act[t, c] = w a sigmoid(slope a) (b + 1), a = min(g, limit), b = clamp(u, -limit, limit), for the channels of ``experts``
+                limit: float, shared_limit: float, slope: float, exact: bool = False, offset: float = 1.0) -> None:
+    """act[t, c] = w a sigmoid(slope a) (b + offset), a = min(g, limit), b = clamp(u, -limit, limit), for the channels of ``experts``
     experts of ``ff`` channels side by side (w = dense[t, expert]) and then ``shared_ff`` channels with w = 1 and a limit of their own."""
     for n, t in (("act", act), ("g", g), ("u", u)):
         _gpu(n, t, act.dtype, 2), _contig(n, t)
@@ -1237,7 +1382,7 @@ def clamped_glu(act: torch.Tensor, g: torch.Tensor, u: torch.Tensor, dense: Opti
         if tuple(dense.shape) != (T, experts):
             raise AlofaError("shape_mismatch", "one weight per row and expert", f"dense={tuple(dense.shape)}")
     _call("alofa_clamped_glu", _ptr(act), _ptr(g), _ptr(u), _I(dtype_code(act)), _ptr(dense if experts else None), _L(T), _I(experts), _I(ff), _I(shared_ff),
-          _F(limit), _F(shared_limit), _F(slope), _I(int(exact)), _stream())
+          _F(limit), _F(shared_limit), _F(slope), _F(offset), _I(int(exact)), _stream())
 
 
 def gemm_channel_scaled(residual: torch.Tensor, a: torch.Tensor, w: torch.Tensor, scale: torch.Tensor, tmp: torch.Tensor, exact: bool = False,
@@ -1270,12 +1415,12 @@ GROUPED_BIG_TILES = 256     # rows of a step from which the many-small-products 
 
 
 def _grouped(out, out_step, x, x_step, w, w2, w_stride, w_step, n_out, K, last, rows, x_by_slot, tiles, tiles_per_batch, tile_batch, row_in,
-             gate, slot_weight, limit, limit_last, slope, epilogue, tile_rows=16) -> None:
+             gate, slot_weight, limit, limit_last, slope, epilogue, tile_rows=16, offset=1.0) -> None:
     last_batch, n_out_last, K_last = last if last is not None else (-1, n_out, K)
     _call("alofa_grouped_product", _ptr(out), _I(dtype_code(out)), _L(_rows("out", out)), _L(out_step), _ptr(x), _L(_rows("x", x)), _L(x_step),
           _ptr(w), _ptr(w2), _L(w_stride), _L(w_step), _I(n_out), _I(K), _I(last_batch), _I(n_out_last), _I(K_last), _I(rows), _I(int(x_by_slot)), _I(tiles),
           _I(tiles_per_batch), _I(tile_rows), _ptr(tile_batch), _ptr(row_in), _ptr(gate), _L(_rows("gate", gate) if gate is not None else 0), _ptr(slot_weight),
-          _F(limit), _F(limit_last), _F(slope), _I(epilogue), _stream())
+          _F(limit), _F(limit_last), _F(slope), _F(offset), _I(epilogue), _stream())
 
 
 def _aligned_rows(t: torch.Tensor) -> bool:
@@ -1336,8 +1481,8 @@ def can_group_experts(x: torch.Tensor, w_gate: torch.Tensor, ff: int, shared_ff:
 
 
 def experts_gate_up(act: torch.Tensor, x: torch.Tensor, w_gate: torch.Tensor, w_up: torch.Tensor, rows: ExpertRows, ff: int, shared_ff: int,
-                    limit: float, shared_limit: float, slope: float) -> None:
-    """act[slot, :] = weight[slot] * a sigmoid(slope a) (b + 1) with a = min(gate_e(x[row]), limit), b = clamp(up_e(x[row]), -limit, limit)
+                    limit: float, shared_limit: float, slope: float, offset: float = 1.0) -> None:
+    """act[slot, :] = weight[slot] * a sigmoid(slope a) (b + offset) with a = min(gate_e(x[row]), limit), b = clamp(up_e(x[row]), -limit, limit)
     for the expert e of the slot; w_gate and w_up hold the experts' matrices one below the other ([E * ff (+ shared_ff), h])."""
     _gpu("act", act, torch.bfloat16, 2), _gpu("x", x, torch.bfloat16, 2), _gpu("w_gate", w_gate, torch.bfloat16, 2), _gpu("w_up", w_up, torch.bfloat16, 2)
     _contig("w_gate", w_gate), _contig("w_up", w_up), _contig("act", act)
@@ -1346,7 +1491,7 @@ def experts_gate_up(act: torch.Tensor, x: torch.Tensor, w_gate: torch.Tensor, w_
     if tuple(w_gate.shape) != (F, h) or tuple(w_up.shape) != (F, h) or act.shape[0] < rows.slots or act.shape[1] < max(ff, shared_ff) or x.shape[0] != rows.T:
         raise AlofaError("shape_mismatch", "the experts' matrices or the slots' rows do not fit", f"act={tuple(act.shape)} x={tuple(x.shape)} w_gate={tuple(w_gate.shape)} F={F}")
     _grouped(act, 0, x, 0, w_gate, w_up, h, ff * h, ff, h, (rows.experts, shared_ff, h) if rows.shared else None, rows.slots, False, rows.tiles, 0,
-             rows.tile_batch, rows.row_in, None, rows.slot_weight, limit, shared_limit, slope, GR_CLAMPED_GLU, rows.tile_rows)
+             rows.tile_batch, rows.row_in, None, rows.slot_weight, limit, shared_limit, slope, GR_CLAMPED_GLU, rows.tile_rows, offset)
 
 
 def experts_down(y: torch.Tensor, act: torch.Tensor, w_down: torch.Tensor, rows: ExpertRows, ff: int, shared_ff: int) -> None:
@@ -1360,8 +1505,11 @@ def experts_down(y: torch.Tensor, act: torch.Tensor, w_down: torch.Tensor, rows:
              rows.tile_batch, rows.row_in, None, None, 0.0, 0.0, 0.0, GR_STORE, rows.tile_rows)
 
 
-def experts_sum(residual: torch.Tensor, y: torch.Tensor, rows: ExpertRows, scale: Optional[torch.Tensor] = None) -> None:
-    """residual[t] += scale * (sum over row t's choices k, ascending, of y[slot of (t, k)], then its slot of the shared expert)."""
+def experts_sum(residual: torch.Tensor, y: torch.Tensor, rows: ExpertRows, scale: Optional[torch.Tensor] = None, passed: Optional[tuple] = None,
+                assign: bool = False) -> None:
+    """residual[t] += scale * (sum over row t's choices k, ascending, of y[slot of (t, k)], then its slot of the shared expert). A choice
+    without a slot (an expert without matrices) adds nothing here; ``passed`` = (weight float32 [T], x bfloat16 [T, h]) adds weight[t] * x[t]
+    to the sum: the row itself, handed on. ``assign``: the sum is stored instead of added."""
     _gpu("residual", residual, torch.float32, 2), _gpu("y", y, torch.float32, 2), _contig("residual", residual), _contig("y", y)
     T, h = residual.shape
     if T != rows.T or tuple(y.shape) != (rows.slots, h):
@@ -1370,4 +1518,11 @@ def experts_sum(residual: torch.Tensor, y: torch.Tensor, rows: ExpertRows, scale
         _gpu("scale", scale, torch.float32, 1), _contig("scale", scale)
         if scale.shape[0] != h:
             raise AlofaError("shape_mismatch", "one factor per channel of the stream", f"scale={tuple(scale.shape)}")
-    _call("alofa_experts_sum", _ptr(residual), _ptr(y), _ptr(rows.slot_of), _ptr(scale), _I(T), _I(h), _I(rows.top), _I(int(rows.shared)), _stream())
+    pw = px = None
+    if passed is not None:
+        pw, px = passed
+        _gpu("pass weight", pw, torch.float32, 1), _contig("pass weight", pw), _gpu("passed rows", px, torch.bfloat16, 2)
+        if pw.shape[0] != T or tuple(px.shape) != (T, h):
+            raise AlofaError("shape_mismatch", "one weight and one row to hand on per row of the stream", f"weight={tuple(pw.shape)} rows={tuple(px.shape)}")
+    _call("alofa_experts_sum", _ptr(residual), _ptr(y), _ptr(rows.slot_of), _ptr(scale), _I(T), _I(h), _I(rows.top), _I(int(rows.shared)),
+          _ptr(pw), _ptr(px), _L(_rows("passed rows", px) if px is not None else 0), _I(int(assign)), _stream())

@@ -9,7 +9,10 @@ scaled_prenorm: a += s0 * mixer(norm0(a)); a += s1 * feed_forward(norm1(a)), wit
 channel, times a factor for all) and an optional feed-forward.
 
 filtered_prenorm: the same as prenorm with a filter over time in front of every sub-layer, an optional feed-forward, and an
-optional weighted average over the outputs of all layers so far."""
+optional weighted average over the outputs of all layers so far.
+
+sandwich: a += post0(mixer(pre0(a))); a += post1(feed_forward(pre1(a))): a norm in front of every sub-layer and one behind it, before
+the sum; the feed-forward optional."""
 from __future__ import annotations
 
 import os
@@ -232,8 +235,59 @@ class ScaledPreNormBlock(Block):
             self._sub_layer(ctx, ff, self.norms[1], self.scales[1], hidden, buf, normed=then is not None)
 
 
+class SandwichBlock(Block):
+    """a += post0(mixer(pre0(a))), then, where the layer has a feed-forward, a += post1(feed_forward(pre1(a))).
+    It reads the layer's parts ``mixer``, ``feed_forward`` (may be None) and ``norms``: (pre0, post0) or (pre0, post0, pre1, post1).
+    Mixer and feed-forward leave their results apart (``out=``); a layer norm behind a sub-layer is applied by the launch that adds
+    to the stream, any other norm runs where the result lies and a sum follows."""
+
+    @classmethod
+    def layer_tensors(cls, layer) -> dict:
+        out = {}
+        for n in layer.part("norms"):
+            out.update(tensors_of("norm", n))
+        out.update(tensors_of("mixer", layer.part("mixer")))
+        if layer.part("feed_forward") is not None:
+            out.update(tensors_of("feed_forward", layer.part("feed_forward")))
+        return out
+
+    def __init__(self, layer, weights, rt):
+        super().__init__(layer, weights, rt)
+        ff = layer.part("feed_forward")
+        norms = layer.part("norms")
+        if len(norms) != (2 if ff is None else 4):
+            raise AlofaError("invalid_argument", "a norm in front of and one behind every sub-layer", f"prefix={layer.prefix} norms={len(norms)} feed_forward={ff is not None}")
+        self.norms = [build_part("norm", n, weights, rt) for n in norms]
+        self.mixer = build_part("mixer", layer.part("mixer"), weights, rt)
+        self.feed_forward = build_part("feed_forward", ff, weights, rt) if ff is not None else None
+        self.parts = [p for p in (*self.norms, self.mixer, self.feed_forward) if p is not None]
+
+    def mixers(self):
+        return self.mixer.stateful_parts()
+
+    def _join(self, hidden, apart, norm):
+        ln = norm.as_layernorm()
+        if ln is not None:
+            ops.layernorm_add(hidden, apart, *ln, exact=self.rt.exact)
+        else:
+            norm.forward(apart, apart)
+            ops.add_scaled(hidden, apart, 1.0, exact=self.rt.exact)
+
+    def forward(self, ctx, entry, hidden):
+        buf = ctx.scratch("normed", tuple(hidden.shape), self.rt.dtype)
+        apart = ctx.scratch("sub_out", tuple(hidden.shape), torch.float32)
+        self.norms[0].forward(buf, hidden)
+        self.mixer.forward(ctx, (entry, 0), buf, hidden, out=apart)
+        self._join(hidden, apart, self.norms[1])
+        if self.feed_forward is not None:
+            self.norms[2].forward(buf, hidden)
+            self.feed_forward.forward(ctx, buf, hidden, out=apart)
+            self._join(hidden, apart, self.norms[3])
+
+
 FUSE_SUMS = os.environ.get("ALOFA_FUSE_SUMS", "1") != "0"      # 0 (for measurements): a scaled sum into the stream and the norm behind it are two launches
 
 register_part("block", "prenorm", PreNormBlock)
 register_part("block", "scaled_prenorm", ScaledPreNormBlock)
 register_part("block", "filtered_prenorm", FilteredPreNormBlock)
+register_part("block", "sandwich", SandwichBlock)

@@ -20,7 +20,7 @@ from .base import PositionEncoding, register_part
 class Rotary(PositionEncoding):
     """params: theta, head_dim, pairing ("half"), dims (how many of a head's first channels are rotated, default all
     of them: channel i < dims/2 is paired with i + dims/2, the angle is p * theta^(-2i/dims), the channels from
-    ``dims`` on pass unchanged).
+    ``dims`` on pass unchanged), factor (every frequency is divided by it: positions stretched linearly; default 1).
 
     The kernels pair channel j with j + head_dim/2. With dims < head_dim the table holds the angle zero for the pairs
     beyond dims/2, and ``channel_order`` names the order of a head's channels in which the design's pairs lie that
@@ -32,6 +32,9 @@ class Rotary(PositionEncoding):
         self.theta = float(spec.params["theta"])
         self.head_dim = int(spec.params["head_dim"])
         self.dims = int(spec.params.get("dims") or self.head_dim)
+        self.factor = float(spec.params.get("factor") or 1.0)
+        if not self.factor > 0:
+            raise AlofaError("invalid_argument", "the factor that stretches positions is positive", f"factor={self.factor}")
         if self.dims <= 0 or self.dims % 2 or self.dims > self.head_dim:
             raise AlofaError("unsupported", "rotated channels: an even count, at most the head's size", f"dims={self.dims} head_dim={self.head_dim}")
         if spec.params.get("pairing", "half") != "half":
@@ -44,6 +47,8 @@ class Rotary(PositionEncoding):
         inv = np.zeros(half, dtype=np.float32)      # (pairs beyond dims/2 keep the angle zero: they pass unchanged)
         for i in range(self.dims // 2):
             inv[i] = np.float32(1.0) / np.float32(math.pow(self.theta, (2.0 * i) / self.dims))
+            if self.factor != 1.0:
+                inv[i] = inv[i] / np.float32(self.factor)
         ang = np.arange(n_positions, dtype=np.float32)[:, None] * inv[None, :]
         ang = ang.astype(np.float32).astype(np.float64)
         return np.cos(ang).astype(np.float32), np.sin(ang).astype(np.float32)
@@ -65,7 +70,7 @@ class Rotary(PositionEncoding):
         """One table per (theta, head size) serves every layer of the model (kept on the runtime).
         A table that has to grow is replaced; the old one is kept alive, since a captured graph
         may still read it (for positions it covers)."""
-        key = ("rotary", self.theta, self.head_dim, self.dims)
+        key = ("rotary", self.theta, self.head_dim, self.dims, self.factor)
         have = self.rt.shared.get(key)
         if have is None or have[0].shape[0] < n_positions:
             n = max(n_positions, 2 * have[0].shape[0] if have else 0)

@@ -11,6 +11,13 @@ time_mix        RWKV-style: each of r, k, v, g, w reads its own mix of the token
                 x + (x' - x) mu_s; w_t = exp(-exp(W_w2 tanh(W_w1 mix_w) + w0)); o_t = (S_(t-1) + diag(u) k_t v_t^T)^T r_t,
                 then the update; o / rms(o) per head, times a weight per channel, times silu(g), output projection.
 
+lightning_attention  w = a constant per head; q, k, v through silu; o_t = S_t^T q_t; the heads together through an RMS norm with a
+                weight, times sigmoid(gate), output projection.
+matrix_memory   exponential gates per head kept in range by a running maximum m (state beside S): i = cap tanh(zi / cap),
+                f = log sigmoid(cap tanh(zf / cap)), m_t = max(f + m_(t-1), i); S_t = exp(f + m_(t-1) - m_t) S_(t-1) + exp(i - m_t) k v^T, a
+                normaliser n_t likewise with k alone; o = S_t^T q / (max(|n_t . q|, exp(-m_t)) + 1e-6), q scaled by dk^(-1/2); o / rms(o)
+                per head, times a weight per channel, times sigmoid(gate), output projection.
+
 Projections and gates run in the activation dtype; decays, the state, the read-out and the head norms in float32.
 Every one of them takes ``out=`` (see ``Mixer.forward``)."""
 from __future__ import annotations
@@ -148,6 +155,115 @@ class GatedLinearAttention(RecurrentMixer):
         self._leave(ctx, o, parts, proj[:, 2 * kd + vd:2 * kd + 2 * vd], self.norm, residual, out)
 
 
+class LightningAttention(RecurrentMixer):
+    """params: prefix, hidden, heads, key_dim, value_dim, decay (one per head), eps. Tensors: prefix + q, k, v, g, o, norm [heads * value_dim]."""
+
+    @classmethod
+    def tensors(cls, spec):
+        p = spec.params
+        pre, h, kd, vd = p["prefix"], p["hidden"], p["heads"] * p["key_dim"], p["heads"] * (p.get("value_dim") or p["key_dim"])
+        return {pre + "q": TensorRule((kd, h), "fan_in"), pre + "k": TensorRule((kd, h), "fan_in"), pre + "v": TensorRule((vd, h), "fan_in"),
+                pre + "g": TensorRule((vd, h), "fan_in"), pre + "o": TensorRule((h, vd), "fan_in"), pre + "norm": TensorRule((vd,), "norm")}
+
+    def __init__(self, spec, weights, rt):
+        super().__init__(spec, weights, rt)
+        p, pre = spec.params, spec.params["prefix"]
+        decay = [float(x) for x in p["decay"]]
+        if len(decay) != self.heads:
+            raise AlofaError("invalid_argument", "one decay per head", f"heads={self.heads} decays={len(decay)}")
+        self.decay = torch.tensor(decay, dtype=torch.float32, device=rt.device)
+        self.w_in = _stacked(rt, [weights[pre + n] for n in ("q", "k", "v", "g")])
+        self.w_o = rt.matrix(weights[pre + "o"])
+        self.norm = rt.vector(weights[pre + "norm"])
+
+    def forward(self, ctx, where, x, residual, out=None):
+        T, kd, vd = x.shape[0], self.heads * self.dk, self.heads * self.dv
+        proj = ctx.scratch("recurrent_proj", (T, 2 * kd + 2 * vd), self.rt.dtype)
+        ops.gemm(proj, x, self.w_in, exact=self.rt.exact)
+        qkv = proj[:, :2 * kd + vd]
+        ops.activation(qkv, qkv, ops.SILU, exact=self.rt.exact)
+        o = self._readouts(ctx, T)
+        parts = ops.linear_recurrence(o, proj[:, :kd], proj[:, kd:2 * kd], proj[:, 2 * kd:2 * kd + vd], ctx.state(where), rows_of_requests(ctx),
+                                      self.heads, self.dk, self.dv, ops.DECAY_PER_HEAD, self.decay)
+        # (the heads together are one row to norm: a "head" of heads * dv channels)
+        y = ctx.scratch("recurrent_gated", (T, vd), self.rt.dtype)
+        ops.headnorm_gate(y, o, proj[:, 2 * kd + vd:], self.norm, 1, vd, self.eps, self.rt.exact, parts=parts, gate_kind="sigmoid")
+        if out is not None:
+            ops.gemm(out, y, self.w_o, exact=self.rt.exact)
+        else:
+            ops.gemm(residual, y, self.w_o, add_to_out=True, exact=self.rt.exact)
+
+
+class GateMaximum(Mixer):
+    """The running maximum of a memory's gates: one float per head and request, beside the memory itself."""
+    capturable = True
+
+    def __init__(self, heads: int, rt):
+        self.heads, self.rt, self.spec = heads, rt, None
+
+    def state_need(self):
+        return StateNeed((self.heads,), torch.float32)
+
+
+class MatrixMemory(RecurrentMixer):
+    """params: prefix, hidden, heads, key_dim, value_dim, gate_cap, eps. Tensors: prefix + q, k, v, g, o, norm [heads * value_dim],
+    i [heads, hidden], i.b [heads], f, f.b.
+
+    The normaliser rides through the recurrence as one more value channel that is always one, so the state of a head is
+    [key_dim, value_dim + 1]; the gates' running maximum is a second piece of state."""
+
+    @classmethod
+    def tensors(cls, spec):
+        p = spec.params
+        H = p["heads"]
+        pre, h, kd, vd = p["prefix"], p["hidden"], H * p["key_dim"], H * (p.get("value_dim") or p["key_dim"])
+        return {pre + "q": TensorRule((kd, h), "fan_in"), pre + "k": TensorRule((kd, h), "fan_in"), pre + "v": TensorRule((vd, h), "fan_in"),
+                pre + "g": TensorRule((vd, h), "fan_in"), pre + "o": TensorRule((h, vd), "fan_in"), pre + "norm": TensorRule((vd,), "norm"),
+                pre + "i": TensorRule((H, h), "fan_in"), pre + "i.b": TensorRule((H,), "bias"), pre + "f": TensorRule((H, h), "fan_in"), pre + "f.b": TensorRule((H,), "gate_bias")}
+
+    def __init__(self, spec, weights, rt):
+        super().__init__(spec, weights, rt)
+        p, pre = spec.params, spec.params["prefix"]
+        self.cap = float(p["gate_cap"])
+        if not self.cap > 0:
+            raise AlofaError("invalid_argument", "the gates' cap is positive", f"gate_cap={self.cap}")
+        self.w_in = _stacked(rt, [weights[pre + n] for n in ("q", "k", "v", "g")])
+        self.w_gates = _stacked(rt, [weights[pre + "i"], weights[pre + "f"]])
+        self.b_gates = rt.vector(torch.cat([weights[pre + "i.b"].float(), weights[pre + "f.b"].float()]))
+        self.w_o = rt.matrix(weights[pre + "o"])
+        self.norm = rt.vector(weights[pre + "norm"])
+        self.q_scale = float(self.dk) ** -0.5
+        self.maximum = GateMaximum(self.heads, rt)
+
+    def state_need(self):
+        return StateNeed((self.heads, self.dk, self.dv + 1), torch.float32)
+
+    def stateful_parts(self):
+        return [self, self.maximum]
+
+    def forward(self, ctx, where, x, residual, out=None):
+        T, H, kd, vd = x.shape[0], self.heads, self.heads * self.dk, self.heads * self.dv
+        entry, k = where if isinstance(where, tuple) else (where, 0)
+        exact, rows = self.rt.exact, rows_of_requests(ctx)
+        proj = ctx.scratch("recurrent_proj", (T, 2 * kd + 2 * vd), self.rt.dtype)
+        ops.gemm(proj, x, self.w_in, exact=exact)
+        z = ctx.scratch("memory_gate_z", (T, 2 * H), torch.float32)
+        ops.gemm(z, x, self.w_gates, self.b_gates, exact=exact)
+        gates = ctx.scratch("memory_gates", (3, T, H), torch.float32)
+        ops.gate_scan(gates, z, ctx.state((entry, k + 1)), rows, H, self.cap)
+        qf, kf = ctx.scratch("memory_q", (T, kd), torch.float32), ctx.scratch("memory_k", (T, kd), torch.float32)
+        vf, decay = ctx.scratch("memory_v", (T, vd + H), torch.float32), ctx.scratch("recurrent_decay", (T, kd), torch.float32)
+        ops.gated_operands(qf, kf, vf, decay, proj[:, :kd], proj[:, kd:2 * kd], proj[:, 2 * kd:2 * kd + vd], gates, H, self.dk, self.dv)
+        o = ctx.scratch("memory_out", (ops.recurrence_max_parts(self.dk), T, vd + H), torch.float32)
+        parts = ops.linear_recurrence(o, qf, kf, vf, ctx.state((entry, k)), rows, H, self.dk, self.dv + 1, ops.DECAY_GIVEN, decay, q_scale=self.q_scale)
+        y = ctx.scratch("recurrent_gated", (T, vd), self.rt.dtype)
+        ops.headnorm_gate(y, o, proj[:, 2 * kd + vd:], self.norm, H, self.dv, self.eps, exact, parts=parts, gate_kind="sigmoid", extra=1, floor=gates[2])
+        if out is not None:
+            ops.gemm(out, y, self.w_o, exact=exact)
+        else:
+            ops.gemm(residual, y, self.w_o, add_to_out=True, exact=exact)
+
+
 MIXES = ("r", "k", "v", "g", "w")
 
 
@@ -282,5 +398,7 @@ class ParallelMixers(Mixer):
 register_part("mixer", "retention", Retention)
 register_part("mixer", "gated_linear", GatedLinearAttention)
 register_part("mixer", "time_mix", TimeMix)
+register_part("mixer", "lightning_attention", LightningAttention)
+register_part("mixer", "matrix_memory", MatrixMemory)
 register_part("mixer", "parallel", ParallelMixers)
 register_part("conv", "token_shift", TokenShift)

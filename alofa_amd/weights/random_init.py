@@ -26,6 +26,8 @@ _DRAWN = {
     "decay_bias": lambda t, shape: t + 2.0,                                    # pre-activations of a sigmoid decay: mostly slow decays
     "log_rate": lambda t, shape: t * 0.5 - 2.0,                                # log of a decay rate: exp(-exp(.)) near 0.87
     "unit_interval": lambda t, shape: torch.sigmoid(t),                        # mixing weights in (0, 1)
+    "head_mix": lambda t, shape: torch.eye(shape[-1], device=t.device) + 0.25 * t,      # heads mixed with one another: mostly themselves
+    "gate_bias": lambda t, shape: t + 1.0,                                     # pre-activations of gates that start open
     "average": lambda t, shape: (1.0 + 0.3 * t) / float(shape[-1]),            # weights of an average over shape[-1] terms
 }
 
