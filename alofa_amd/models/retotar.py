@@ -165,7 +165,7 @@ class RetotarConfig(ModelConfig):
         return PartSpec("routed_experts", {
             "prefix": pre, "hidden": self.width, "experts": r["experts"], "top": r["top"], "score": "softmax", "correction": "correction",
             "groups": r.get("groups"), "passing": r["identity"], "renormalize": False, "expert": {"intermediate": mlp["expert"]["ff"]}, "shared": None,
-            "activation": "silu_glu", "names": {"router": "router", "expert": "e{}", "shared": "shared", "gate": "gate", "up": "up", "down": "down"}})
+            "activation": "silu_glu", "router_init": "decisive", "names": {"router": "router", "expert": "e{}", "shared": "shared", "gate": "gate", "up": "up", "down": "down"}})
 
     def spec(self) -> ModelSpec:
         h = self.width

@@ -32,7 +32,7 @@ class RoutedExperts(FeedForward):
     shared (the same, or None), activation ("clamped_glu"), slope, names (after the prefix: router; expert, a pattern with {}
     for the expert's number; shared; gate, up, down after an expert's name and a dot).
     Optional: correction (a tensor's name after the prefix, [experts + passing]), groups {count, keep}, passing (experts without
-    matrices behind the others; the router has experts + passing outputs).
+    matrices behind the others; the router has experts + passing outputs), router_init (the rule random router weights are drawn by).
     ``forward(..., scale=)`` with a float32 vector: what is added to the stream is multiplied by it channel by channel;
     ``forward(..., out=)``: the result is stored there (float32, the stream's shape) and the stream left alone."""
     capturable = True
@@ -52,7 +52,7 @@ class RoutedExperts(FeedForward):
         for e in range(p["experts"]):
             names, i = cls._expert_names(p, e), p["expert"]["intermediate"]
             out.update({names["gate"]: TensorRule((i, h), "fan_in"), names["up"]: TensorRule((i, h), "fan_in"), names["down"]: TensorRule((h, i), "fan_in")})
-        out[p["prefix"] + p["names"]["router"]] = TensorRule((p["experts"] + int(p.get("passing", 0)), h), "fan_in")
+        out[p["prefix"] + p["names"]["router"]] = TensorRule((p["experts"] + int(p.get("passing", 0)), h), p.get("router_init", "fan_in"))
         if p.get("correction") is not None:
             out[p["prefix"] + p["correction"]] = TensorRule((p["experts"] + int(p.get("passing", 0)),), "bias")
         if p.get("shared") is not None:

@@ -28,6 +28,7 @@ _DRAWN = {
     "unit_interval": lambda t, shape: torch.sigmoid(t),                        # mixing weights in (0, 1)
     "head_mix": lambda t, shape: torch.eye(shape[-1], device=t.device) + 0.25 * t,      # heads mixed with one another: mostly themselves
     "gate_bias": lambda t, shape: t + 1.0,                                     # pre-activations of gates that start open
+    "decisive": lambda t, shape: t * 8.0 / float(shape[-1]) ** 0.5,           # a router whose calls are seldom close
     "average": lambda t, shape: (1.0 + 0.3 * t) / float(shape[-1]),            # weights of an average over shape[-1] terms
 }
 

@@ -113,3 +113,16 @@ def rerupel_dirs(tmp_path_factory):
         write_random_model(cfg, d, seed=3000 + ord(name))
         out[name] = d
     return out
+
+
+@pytest.fixture(scope="session")
+def retotar_dirs(tmp_path_factory):
+    """Model folders of the small Retotar configurations, written by the engine's random-weights mode."""
+    from alofa_amd.weights import write_random_model
+    from retotar_cases import RETOTAR
+    out = {}
+    for name, cfg in RETOTAR.items():
+        d = tmp_path_factory.mktemp(f"retotar_{name}")
+        write_random_model(cfg, d, seed=4000 + ord(name))
+        out[name] = d
+    return out

@@ -5,8 +5,6 @@ nothing with the engine; the tests compare the engine's logits (and its residual
 ``store``: optional function applied to what a bfloat16 engine keeps rounded between kernels (see ``rounder``)."""
 from __future__ import annotations
 
-import math
-
 import torch
 
 F = torch.float64
@@ -29,10 +27,6 @@ def layer_norm(x, w, b, eps):
 
 def unit_rms(x, eps):
     return x / torch.sqrt((x * x).mean(-1, keepdim=True) + eps)
-
-
-def gelu_tanh(z):
-    return 0.5 * z * (1 + torch.tanh(math.sqrt(2 / math.pi) * (z + 0.044715 * z ** 3)))
 
 
 def silu(z):
@@ -205,3 +199,96 @@ def forward(cfg, weights, tokens, store=_id, layers_out=None):
             layers_out.append(x.clone())
     y = store(norm("final.norm", x))
     return y @ weights["head"].to(F).T
+
+
+# ---- for the tests: folders, logits as arrays, how close the routers' calls are, greedy continuation
+
+def read_config(model_dir):
+    import json
+    from pathlib import Path
+    return json.loads((Path(model_dir) / "config.json").read_text())
+
+
+def read_weights(model_dir):
+    from pathlib import Path
+    from safetensors.torch import load_file
+    return {k: v.to(F) for k, v in load_file(str(Path(model_dir) / "model.safetensors")).items()}
+
+
+def to_bfloat16(x):
+    return x.to(torch.bfloat16).to(F)
+
+
+def forward_logits(weights, cfg, tokens, store=_id):
+    return forward(cfg, weights, tokens, store).numpy()
+
+
+def forward_hidden(weights, cfg, tokens):
+    out = []
+    forward(cfg, weights, tokens, layers_out=out)
+    return [x.numpy() for x in out]
+
+
+def router_margins(weights, cfg, tokens):
+    """Per position the smallest gap, over all layers, between what a router takes and what it leaves (experts and groups), relative to
+    the scores that a change of the router's input would move."""
+    eps = cfg["norm"]["eps"]
+    T = len(tokens)
+    margins = torch.full((T,), float("inf"), dtype=F)
+    seen = []
+    forward(cfg, weights, tokens, layers_out=seen)
+    ids = torch.as_tensor(tokens, dtype=torch.long)
+    x0 = weights["embed"].to(F)[ids] * cfg["embedding"]["scale"]
+    for i, layer in enumerate(cfg["layers"]):
+        if layer.get("mlp") is None:
+            continue
+        # the stream in front of the feed-forward: the layer's output minus what the feed-forward added is not kept, so it is made again
+        p = f"l{i}."
+        before = x0 if i == 0 else seen[i - 1]
+        W = _sub(weights, p + "mix.")
+        h = layer_norm(before, weights[p + "norm1"].to(F), weights[p + "norm1.b"].to(F), eps)
+        m = layer["mixer"]
+        if layer["type"] == "attention":
+            src = m.get("kv_from")
+            if src is None:
+                kv = attention_keys_values(h, W, m, eps)
+            else:
+                prev = x0 if src == 0 else seen[src - 1]
+                hs = layer_norm(prev, weights[f"l{src}.norm1"].to(F), weights[f"l{src}.norm1.b"].to(F), eps)
+                kv = attention_keys_values(hs, _sub(weights, f"l{src}.mix."), cfg["layers"][src]["mixer"], eps)
+            y = attention(h, W, m, eps, kv)
+        elif layer["type"] == "lightning":
+            y = lightning(h, W, m, eps)
+        else:
+            y = mlstm(h, W, m, eps)
+        x = before + layer_norm(y, weights[p + "norm1b"].to(F), weights[p + "norm1b.b"].to(F), eps)
+        h2 = layer_norm(x, weights[p + "norm2"].to(F), weights[p + "norm2.b"].to(F), eps)
+        r = layer["mlp"]["router"]
+        Wm = _sub(weights, p + "mlp.")
+        s = torch.softmax(h2 @ Wm["router"].to(F).T, dim=-1)
+        c = s + Wm["correction"].to(F)
+        groups = r.get("groups") or {"count": 1, "keep": 1}
+        size = c.shape[1] // groups["count"]
+        best = c.view(T, groups["count"], size).max(-1).values
+        # a gap between two choice scores counts against the softmax scores behind them: those are what a small change of z moves
+        order = best.sort(-1, descending=True)
+        if groups["keep"] < groups["count"]:
+            at = c.view(T, groups["count"], size).argmax(-1) + torch.arange(groups["count"]) * size      # the member behind a group's score
+            s_best = torch.gather(torch.gather(s, 1, at), 1, order.indices)
+            gap = order.values[:, groups["keep"] - 1] - order.values[:, groups["keep"]]
+            margins = torch.minimum(margins, gap / (s_best[:, groups["keep"] - 1] + s_best[:, groups["keep"]]))
+        kept = order.indices[:, :groups["keep"]]
+        allowed = torch.zeros_like(best, dtype=torch.bool).scatter_(1, kept, True).repeat_interleave(size, dim=1)
+        ca = c.masked_fill(~allowed, float("-inf")).sort(-1, descending=True)
+        if r["top"] < int(allowed[0].sum()):
+            sa = torch.gather(s, 1, ca.indices)
+            gap = ca.values[:, r["top"] - 1] - ca.values[:, r["top"]]
+            margins = torch.minimum(margins, gap / (sa[:, r["top"] - 1] + sa[:, r["top"]]))
+    return margins.numpy()
+
+
+def greedy(weights, cfg, prompt, n_new):
+    ids = list(prompt)
+    for _ in range(n_new):
+        ids.append(int(forward(cfg, weights, ids)[-1].argmax()))
+    return ids[len(prompt):]
