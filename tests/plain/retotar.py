@@ -37,8 +37,12 @@ def turn_halves(x, pos, n, base, factor=1.0, sign=1.0):
     """The first ``n`` channels of the last axis turned by the positions' angles: channel i pairs with i + n/2, the angle
     of pair i is pos * base^(-2i/n) / factor; the rest passes. x [T, heads, d], pos [T]."""
     half = n // 2
-    f = torch.tensor([base ** (-2.0 * i / n) / factor for i in range(half)], dtype=F)
-    a = sign * pos.to(F)[:, None, None] * f[None, None, :]
+    # (frequencies and angles are 32-bit numbers in this design: the angle of a far position is known to some 1e-5 only, and a twin that
+    # knew it better would differ from every engine by that much)
+    f = torch.tensor(1.0, dtype=torch.float32) / torch.tensor([base ** (2.0 * i / n) for i in range(half)], dtype=F).to(torch.float32)
+    if factor != 1.0:
+        f = f / torch.tensor(factor, dtype=torch.float32)
+    a = sign * (pos.to(torch.float32)[:, None, None] * f[None, None, :]).to(F)
     u, v = x[..., :half], x[..., half:n]
     return torch.cat([u * torch.cos(a) - v * torch.sin(a), v * torch.cos(a) + u * torch.sin(a), x[..., n:]], dim=-1)
 
