@@ -28,7 +28,7 @@ context of 4,096) through the same engine and print their own line;
 ``--config 1.5b``, ``3b`` and ``14b`` run the continuous batch at those sizes.
 ``--sweep batch`` and ``--sweep context`` take any of the configurations.
 
-``--design tugalix`` and ``--design rerupel`` measure another design beside Qwen2 at equal sizes: prefill of one prompt and
+``--design tugalix``, ``--design rerupel`` and ``--design retotar`` measure another design beside Qwen2 (Retotar: beside Tugalix) at equal sizes: prefill of one prompt and
 decode steps at batch 1, 8 and 64, at a few widths (``--sizes``), a line per point and model."""
 import argparse
 import json
@@ -526,7 +526,31 @@ def rerupel_sizes(width, heads, dim, ff, layers, vocab=32000):
     return rer, qwen
 
 
-DESIGN_MODELS = {"tugalix": tugalix_sizes, "rerupel": rerupel_sizes}
+def retotar_sizes(width, heads, dim, ff, layers, vocab=32000):
+    """A Retotar model of ``layers`` layers in the order attention (a window of 1,024 keys), lightning, mlstm, attention that reads the
+    first one's pages, every one with sixteen experts of which a token takes four (two identity experts beside them, two groups of which
+    one is kept), and beside it the closest other design, Tugalix, at equal width, heads and layers, with a dense feed-forward of as many
+    weights as a token's four experts."""
+    kv = max(1, heads // 4)
+    expert = max(64, ff // 8 // 64 * 64)
+    rot = {"dims": dim // 2, "base": 1000000.0, "scaling": {"factor": 8.0}}
+    attention = {"heads": heads, "kv_heads": kv, "dim": dim, "vdim": dim, "rot": rot, "scale": 8.0 / dim, "mask": {"size": 1024}}
+    moe = {"kind": "moe", "router": {"experts": 16, "top": 4, "identity": 2, "groups": {"count": 2, "keep": 1}}, "expert": {"ff": expert}}
+
+    def mixer(i):
+        k = i % 4
+        if k == 1:
+            return "lightning", {"heads": heads, "dim": dim, "vdim": dim, "decay": [1.0 - 2.0 ** (-5 - h % 8) for h in range(heads)]}
+        if k == 2:
+            return "mlstm", {"heads": heads, "dim": dim, "vdim": dim, "gate_cap": 15.0}
+        return "attention", dict(attention, kv_from=i - 3) if k == 3 else dict(attention)
+    ret = {"architecture": "Retotar", "vocab": vocab, "width": width, "norm": {"eps": 1e-5}, "embedding": {"scale": 1.0},
+           "layers": [{"type": mixer(i)[0], "mixer": mixer(i)[1], "mlp": moe} for i in range(layers)]}
+    return ret, tugalix_sizes(width, heads, dim, 6 * expert, layers, vocab)[0]
+
+
+DESIGN_MODELS = {"tugalix": tugalix_sizes, "rerupel": rerupel_sizes, "retotar": retotar_sizes}
+DESIGN_BESIDE = {"retotar": "tugalix"}      # the model a design is measured beside, where that is not Qwen2
 DESIGN_SIZES = {"256": (256, 4, 64, 1024, 4), "1k": (1024, 16, 64, 4096, 8), "2k": (2048, 16, 128, 8192, 8), "4k": (4096, 32, 128, 14336, 4)}
 DESIGN_DEFAULT = ("1k", "2k", "4k")      # ("256": a small one, for a quick look)
 
@@ -539,7 +563,7 @@ def designs(args):
         if size not in DESIGN_SIZES:
             print(f"no such size: {size} (known: {','.join(DESIGN_SIZES)})")
             return 2
-        for name, cfg in zip((args.design, "qwen2"), DESIGN_MODELS[args.design](*DESIGN_SIZES[size])):
+        for name, cfg in zip((args.design, DESIGN_BESIDE.get(args.design, "qwen2")), DESIGN_MODELS[args.design](*DESIGN_SIZES[size])):
             if args.only and name != args.only:
                 continue
             cfg = dict(cfg, vocab_size=cfg.get("vocab_size", cfg.get("vocab")))      # (the points draw their tokens by this key)
