@@ -44,6 +44,12 @@ typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 
 constexpr int kMaxSplits = 64;
+
+// A result goes to the bfloat16 rows, or, where `out32` is given, unrounded to float rows of the same shape.
+__device__ __forceinline__ void put_out(bf16_t* out, float* out32, int64_t at, float v) {
+  if (out32) out32[at] = v;
+  else store_f32(out + at, v);
+}
 constexpr int kHeadsPerBlock = 16;   // query heads of one key head that a block serves (the columns of a tile)
 
 // What the kernel needs to take the new token's projections as they come out of the fused query / key / value
@@ -86,7 +92,7 @@ __global__ void __launch_bounds__(64 * NW) attention_decode_kernel(
     int64_t q_stride, bf16_t* __restrict__ k_cache, bf16_t* __restrict__ v_cache,
     const int32_t* __restrict__ block_table, int max_blocks, const int32_t* __restrict__ req_of_token,
     const int32_t* __restrict__ positions, const int32_t* __restrict__ rows, int heads, int kv_heads,
-    int bs_shift, int window, float scale, RopeArgs rope, int* __restrict__ counters) {
+    int bs_shift, int window, float scale, RopeArgs rope, int* __restrict__ counters, int v_head, float* __restrict__ out32) {
   static_assert(!kRope || DT % 4 == 0, "the rotation needs a channel and its partner in the same lane: d a multiple of 64");
   constexpr int d = DT * 16;
   constexpr int DS = (d + 31) / 32;            // steps of 32 along d in the first product
@@ -98,6 +104,7 @@ __global__ void __launch_bounds__(64 * NW) attention_decode_kernel(
   // the tokens served are rows[0..gridDim.x) of the packed batch, or all of it
   const int t = rows ? rows[blockIdx.x] : blockIdx.x;
   const int hk = blockIdx.y / chunks, h0 = (blockIdx.y % chunks) * kHeadsPerBlock;
+  const int hv = v_head >= 0 ? v_head : hk;      // the value head whose values the weights meet (v_head >= 0: one for all key heads)
   const int wave = threadIdx.x / 64, lane = threadIdx.x % 64;
   const int c16 = lane % 16, g = lane / 16;
   const int n_parts = gridDim.z, n_splits = n_parts * NW, split = blockIdx.z * NW + wave;
@@ -198,7 +205,7 @@ __global__ void __launch_bounds__(64 * NW) attention_decode_kernel(
       }
 #pragma unroll
       for (int nt = 0; nt < DT; ++nt)
-        s.v[kt][nt] = *reinterpret_cast<const uint2*>(v_cache + ((((vblk * kv_heads + hk) * d + nt * 16 + c16) << bs_shift) + (key4 & bs_mask)));
+        s.v[kt][nt] = *reinterpret_cast<const uint2*>(v_cache + ((((vblk * kv_heads + hv) * d + nt * 16 + c16) << bs_shift) + (key4 & bs_mask)));
     }
   };
 
@@ -379,7 +386,7 @@ __global__ void __launch_bounds__(64 * NW) attention_decode_kernel(
       acc += state[w][i][4 + c] * e;
     }
     if (n_parts == 1) {
-      store_f32(out + static_cast<int64_t>(t) * out_stride + static_cast<int64_t>(h) * d + c, acc / total);
+      put_out(out, out32, static_cast<int64_t>(t) * out_stride + static_cast<int64_t>(h) * d + c, acc / total);
     } else {
       float* dst = partial + ((static_cast<int64_t>(blockIdx.x) * heads + h) * n_parts + blockIdx.z) * (d + 2);
       if (counters) {   // (device scope: written through to memory, where blocks on every die find it)
@@ -455,7 +462,7 @@ __global__ void __launch_bounds__(64 * NW) attention_decode_kernel(
         acc += __hip_atomic_load(part + 2 + c, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) * e;
       }
     }
-    store_f32(out + static_cast<int64_t>(t) * out_stride + static_cast<int64_t>(h) * d + c, acc / total);
+    put_out(out, out32, static_cast<int64_t>(t) * out_stride + static_cast<int64_t>(h) * d + c, acc / total);
   }
 }
 
@@ -467,7 +474,7 @@ __global__ void __launch_bounds__(64 * NW) attention_decode_kernel(
 __global__ void __launch_bounds__(256) attention_merge_kernel(bf16_t* __restrict__ out, int64_t out_stride,
                                                               const float* __restrict__ partial,
                                                               const int32_t* __restrict__ rows, int heads, int d,
-                                                              int n_splits) {
+                                                              int n_splits, float* __restrict__ out32) {
   __shared__ float sums[4][256];
   const int t = rows ? rows[blockIdx.x] : blockIdx.x, h = blockIdx.y, lane = threadIdx.x % 64;
   const int wave = threadIdx.x / 64, waves = blockDim.x / 64;
@@ -503,7 +510,7 @@ __global__ void __launch_bounds__(256) attention_merge_kernel(bf16_t* __restrict
         for (int w = 1; w < waves; ++w) acc += sums[w][c < d ? c : 0];
       }
     }
-    if (wave == 0 && c < d) store_f32(out + static_cast<int64_t>(t) * out_stride + static_cast<int64_t>(h) * d + c, acc / total);
+    if (wave == 0 && c < d) put_out(out, out32, static_cast<int64_t>(t) * out_stride + static_cast<int64_t>(h) * d + c, acc / total);
   }
 }
 
@@ -533,12 +540,15 @@ extern "C" int alofa_attention_decode_can_hand_over(int tokens, int heads, int k
 // q holds rows [queries | keys | values] of one new token per request. req_of_token may be null when every
 // request brings one token: token i then belongs to row i of block_table. hand_over: the parts meet in the
 // workspace (alofa_attention_decode_can_hand_over must hold; `partial` is not used), not in `partial` and a second kernel.
-extern "C" int alofa_attention_decode(void* out, int64_t out_stride, float* partial, const void* q, int64_t q_stride,
-                                      void* k_cache, void* v_cache, const int32_t* block_table,
-                                      int max_blocks, const int32_t* req_of_token, const int32_t* positions,
-                                      const int32_t* rows, int tokens, int heads, int kv_heads, int d, int block_size, int window,
-                                      float scale, int n_splits, const float* cos_t, const float* sin_t, const int64_t* slots,
-                                      int hand_over, hipStream_t stream) {
+// v_head >= 0: every query head's weights meet the values of that one value head (its keys stay its own key head's);
+// out32: the results go there unrounded, as float rows of `out`'s shape and stride, and `out` is not written.
+extern "C" int alofa_attention_decode_v(void* out, int64_t out_stride, float* partial, const void* q, int64_t q_stride,
+                                        void* k_cache, void* v_cache, const int32_t* block_table,
+                                        int max_blocks, const int32_t* req_of_token, const int32_t* positions,
+                                        const int32_t* rows, int tokens, int heads, int kv_heads, int d, int block_size, int window,
+                                        float scale, int n_splits, const float* cos_t, const float* sin_t, const int64_t* slots,
+                                        int hand_over, int v_head, float* out32, hipStream_t stream) {
+  ALOFA_REQUIRE(v_head < kv_heads && (v_head < 0 || !cos_t), "attention_decode: value head %d of %d (and none with the rotary variant)", v_head, kv_heads);
   ALOFA_REQUIRE(tokens > 0 && heads > 0 && kv_heads > 0 && heads % kv_heads == 0,
                 "attention_decode: tokens=%d heads=%d kv_heads=%d (kv_heads must divide heads)", tokens, heads, kv_heads);
   ALOFA_REQUIRE(d >= 16 && d <= 256 && d % 16 == 0, "attention_decode: head size %d must be 16..256 in steps of 16", d);
@@ -567,7 +577,7 @@ extern "C" int alofa_attention_decode(void* out, int64_t out_stride, float* part
   attention_decode_kernel<DT, NW, ROPE><<<grid, 64 * NW, 0, stream>>>(                                                    \
       static_cast<bf16_t*>(out), out_stride, partial, static_cast<const bf16_t*>(q), q_stride,                            \
       static_cast<bf16_t*>(k_cache), static_cast<bf16_t*>(v_cache), block_table, max_blocks, req_of_token,                \
-      positions, rows, heads, kv_heads, bs_shift, window, scale, rope, counters)
+      positions, rows, heads, kv_heads, bs_shift, window, scale, rope, counters, v_head, out32)
   if (fused) {
     switch (d / 64) {
       case 1: ALOFA_DECODE(4, 8, true); break;
@@ -599,8 +609,18 @@ extern "C" int alofa_attention_decode(void* out, int64_t out_stride, float* part
   if (check_launch("attention_decode")) return 1;
   if (n_splits > 1 && !counters) {
     // (one wave up to sixteen parts, whose loads are all on their way at once; four beyond)
-    attention_merge_kernel<<<dim3(tokens, heads), n_splits <= 16 ? 64 : 256, 0, stream>>>(static_cast<bf16_t*>(out), out_stride, partial, rows, heads, d, n_splits);
+    attention_merge_kernel<<<dim3(tokens, heads), n_splits <= 16 ? 64 : 256, 0, stream>>>(static_cast<bf16_t*>(out), out_stride, partial, rows, heads, d, n_splits, out32);
     return check_launch("attention_merge");
   }
   return 0;
+}
+
+extern "C" int alofa_attention_decode(void* out, int64_t out_stride, float* partial, const void* q, int64_t q_stride,
+                                      void* k_cache, void* v_cache, const int32_t* block_table,
+                                      int max_blocks, const int32_t* req_of_token, const int32_t* positions,
+                                      const int32_t* rows, int tokens, int heads, int kv_heads, int d, int block_size, int window,
+                                      float scale, int n_splits, const float* cos_t, const float* sin_t, const int64_t* slots,
+                                      int hand_over, hipStream_t stream) {
+  return alofa_attention_decode_v(out, out_stride, partial, q, q_stride, k_cache, v_cache, block_table, max_blocks, req_of_token, positions, rows, tokens,
+                                  heads, kv_heads, d, block_size, window, scale, n_splits, cos_t, sin_t, slots, hand_over, -1, nullptr, stream);
 }

@@ -65,7 +65,7 @@ __global__ void __launch_bounds__(64 * WPT * TEAMS, (RW == 32 && 64 * WPT * TEAM
     bf16_t* __restrict__ out, int64_t out_stride, const bf16_t* __restrict__ q, int64_t q_stride,
     const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache, const int32_t* __restrict__ block_table,
     int max_blocks, const int32_t* __restrict__ tiles, int heads, int kv_heads, int bs_shift, int window,
-    float scale) {
+    float scale, int v_head, float* __restrict__ out32) {
   constexpr int d = DT * 16;
   constexpr int BKV = KT;
   static_assert(KT == 64 || (KT == 32 && RW == 32), "tiles of 64 keys, or of 32 with 32 rows a wave");
@@ -96,6 +96,7 @@ __global__ void __launch_bounds__(64 * WPT * TEAMS, (RW == 32 && 64 * WPT * TEAM
   const int hk = kShare ? blockIdx.y / chunks : blockIdx.y / group;
   const bool head_ok = !kShare || (blockIdx.y % chunks) * WPT + wave < group;
   const int head = kShare ? hk * group + (head_ok ? (blockIdx.y % chunks) * WPT + wave : 0) : blockIdx.y;
+  const int hv = v_head >= 0 ? v_head : hk;      // the value head whose values the weights meet (v_head >= 0: one for all key heads)
   for (int part = 0; part < 2; ++part) {
   const int32_t* tile = tiles + 8 * blockIdx.x + 4 * part;
   // kShare: the block takes rows RW z .. of the run (fewer at the run's end; none: the block has nothing to do in this run)
@@ -172,7 +173,7 @@ __global__ void __launch_bounds__(64 * WPT * TEAMS, (RW == 32 && 64 * WPT * TEAM
       const int c = chunk_of(j);
       const int key0 = clamp(v_key0(t, j), v_first, v_last), channel = c / (BKV / 8);
       v_reg[j] = *reinterpret_cast<const uint4*>(
-          v_cache + (((static_cast<int64_t>(v_page[j]) * kv_heads + hk) * d + channel) << bs_shift) + (key0 & page_mask));
+          v_cache + (((static_cast<int64_t>(v_page[j]) * kv_heads + hv) * d + channel) << bs_shift) + (key0 & page_mask));
     }
   };
   // With 32 rows a wave the next tile's values are asked for only once this tile's scores have become weights:
@@ -426,7 +427,8 @@ __global__ void __launch_bounds__(64 * WPT * TEAMS, (RW == 32 && 64 * WPT * TEAM
   }
   if (row_ok && team == 0) {
     const float inv = 1.f / l;
-    bf16_t* dst = out + static_cast<int64_t>(row0 + my_row) * out_stride + static_cast<int64_t>(head) * d;
+    const int64_t at = static_cast<int64_t>(row0 + my_row) * out_stride + static_cast<int64_t>(head) * d;
+    bf16_t* dst = out + at;
 #pragma unroll
     for (int nt = 0; nt < OT; ++nt) {
 #pragma unroll
@@ -435,7 +437,9 @@ __global__ void __launch_bounds__(64 * WPT * TEAMS, (RW == 32 && 64 * WPT * TEAM
         w.x = pack_bf16x2(o[nt][4 * j] * inv, o[nt][4 * j + 1] * inv);
         w.y = pack_bf16x2(o[nt][4 * j + 2] * inv, o[nt][4 * j + 3] * inv);
         const int c = RW == 32 ? nt * 32 + 8 * j + 4 * h : nt * 16 + g * 4;
-        if (RW == 16 || c < d) *reinterpret_cast<uint2*>(dst + c) = w;
+        if (out32) {      // unrounded, to float rows of the same shape (uniform over the launch)
+          if (RW == 16 || c < d) *reinterpret_cast<float4*>(out32 + at + c) = make_float4(o[nt][4 * j] * inv, o[nt][4 * j + 1] * inv, o[nt][4 * j + 2] * inv, o[nt][4 * j + 3] * inv);
+        } else if (RW == 16 || c < d) *reinterpret_cast<uint2*>(dst + c) = w;
       }
     }
   }
@@ -498,10 +502,13 @@ extern "C" int alofa_attention_prefill_supports(int d) {
   return d == 16 || d == 32 || d == 48 || d == 64 || d == 96 || d == 128 || d == 256;
 }
 
-extern "C" int alofa_attention_prefill(void* out, int64_t out_stride, const void* q, int64_t q_stride,
-                                       const void* k_cache, const void* v_cache, const int32_t* block_table,
-                                       int max_blocks, const int32_t* tiles, int n_tiles, int heads, int kv_heads, int d,
-                                       int block_size, int window, float scale, int share, int rows_per_wave, hipStream_t stream) {
+// v_head >= 0: every query head's weights meet the values of that one value head (its keys stay its own key head's);
+// out32: the results go there unrounded, as float rows of `out`'s shape and stride (16-byte aligned), and `out` is not written.
+extern "C" int alofa_attention_prefill_v(void* out, int64_t out_stride, const void* q, int64_t q_stride,
+                                         const void* k_cache, const void* v_cache, const int32_t* block_table,
+                                         int max_blocks, const int32_t* tiles, int n_tiles, int heads, int kv_heads, int d,
+                                         int block_size, int window, float scale, int share, int rows_per_wave, int v_head, float* out32, hipStream_t stream) {
+  ALOFA_REQUIRE(v_head < kv_heads && reinterpret_cast<uintptr_t>(out32) % 16 == 0, "attention_prefill: value head %d of %d; float rows 16-byte aligned", v_head, kv_heads);
   ALOFA_REQUIRE(n_tiles > 0 && heads > 0 && kv_heads > 0 && heads % kv_heads == 0,
                 "attention_prefill: tiles=%d heads=%d kv_heads=%d (kv_heads must divide heads)", n_tiles, heads, kv_heads);
   ALOFA_REQUIRE(alofa_attention_prefill_supports(d), "attention_prefill: head size %d is not built (16, 32, 48, 64, 96, 128, 256 are)", d);
@@ -522,11 +529,11 @@ extern "C" int alofa_attention_prefill(void* out, int64_t out_stride, const void
 #define ALOFA_PREFILL_AS(DT, TEAMS, WPT, SHARE, GRID)                                                                         \
   attention_prefill_kernel<DT, TEAMS, WPT, SHARE><<<GRID, 64 * WPT * TEAMS, 0, stream>>>(                                    \
       static_cast<bf16_t*>(out), out_stride, static_cast<const bf16_t*>(q), q_stride, static_cast<const bf16_t*>(k_cache), \
-      static_cast<const bf16_t*>(v_cache), block_table, max_blocks, tiles, heads, kv_heads, bs_shift, window, scale)
+      static_cast<const bf16_t*>(v_cache), block_table, max_blocks, tiles, heads, kv_heads, bs_shift, window, scale, v_head, out32)
 #define ALOFA_PREFILL_AS32(DT, TEAMS, WPT, SHARE, GRID)                                                                       \
   attention_prefill_kernel<DT, TEAMS, WPT, SHARE, 32, (DT > 6 ? 32 : 64)><<<GRID, 64 * WPT * TEAMS, 0, stream>>>(            \
       static_cast<bf16_t*>(out), out_stride, static_cast<const bf16_t*>(q), q_stride, static_cast<const bf16_t*>(k_cache), \
-      static_cast<const bf16_t*>(v_cache), block_table, max_blocks, tiles, heads, kv_heads, bs_shift, window, scale)
+      static_cast<const bf16_t*>(v_cache), block_table, max_blocks, tiles, heads, kv_heads, bs_shift, window, scale, v_head, out32)
 #define ALOFA_PREFILL_WIDE32(DT, WPT)                                                                            \
   if (width == WPT) ALOFA_PREFILL_AS32(DT, (kShareTeams<DT>), WPT, true, dim3(n_tiles, kv_heads * chunks, 2))
 #define ALOFA_PREFILL32(DT)                                                                         \
@@ -561,4 +568,12 @@ extern "C" int alofa_attention_prefill(void* out, int64_t out_stride, const void
 #undef ALOFA_PREFILL_AS32
 #undef ALOFA_PREFILL_AS
   return check_launch("attention_prefill");
+}
+
+extern "C" int alofa_attention_prefill(void* out, int64_t out_stride, const void* q, int64_t q_stride,
+                                       const void* k_cache, const void* v_cache, const int32_t* block_table,
+                                       int max_blocks, const int32_t* tiles, int n_tiles, int heads, int kv_heads, int d,
+                                       int block_size, int window, float scale, int share, int rows_per_wave, hipStream_t stream) {
+  return alofa_attention_prefill_v(out, out_stride, q, q_stride, k_cache, v_cache, block_table, max_blocks, tiles, n_tiles, heads, kv_heads, d, block_size, window,
+                                   scale, share, rows_per_wave, -1, nullptr, stream);
 }

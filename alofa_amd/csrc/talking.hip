@@ -10,7 +10,7 @@
 //                     values of its own key/value head; the result is turned back by the row's own position (values were
 //                     turned by theirs), and optionally multiplied by the sigmoid of a gate.
 //
-// Cache layout (this part's own): keys [block, kv_head, slot, d], values [block, kv_head, slot, dv]; d and dv may differ.
+// Cache layout (that of the other attention kernels): keys [block, kv_head, slot, d], values transposed [block, kv_head, dv, slot]; d and dv may differ.
 //
 // Arithmetic: products and sums in Acc (float; double in the exact path), in ascending key order per output channel, so a
 // row's result depends on the keys it sees and on nothing else: not on how rows were cut into steps, on the batch or on pages.
@@ -37,11 +37,14 @@ __global__ void __launch_bounds__(256) turn_norm_write_kernel(T* __restrict__ qk
   const int width = is_v ? dv : d, half = is_v ? dv / 2 : half_qk;
   T* src = qkv + static_cast<int64_t>(t) * stride + (is_v ? static_cast<int64_t>(heads + kv_heads) * d + static_cast<int64_t>(u - heads - kv_heads) * dv : static_cast<int64_t>(u) * d);
   T* dst = src;
-  if (is_k || is_v) {
+  int64_t step = 1;      // between two channels at the destination (values lie transposed in their pages: a channel's slots side by side)
+  if (is_k) {
     const int64_t slot = slots[t];
-    const int c = is_v ? u - heads - kv_heads : u - heads;
-    T* cache = is_v ? v_cache : k_cache;
-    dst = cache + (((slot / block_size) * kv_heads + c) * block_size + slot % block_size) * static_cast<int64_t>(width);
+    dst = k_cache + (((slot / block_size) * kv_heads + (u - heads)) * block_size + slot % block_size) * static_cast<int64_t>(d);
+  } else if (is_v) {
+    const int64_t slot = slots[t];
+    dst = v_cache + ((slot / block_size) * kv_heads + (u - heads - kv_heads)) * static_cast<int64_t>(dv) * block_size + slot % block_size;
+    step = block_size;
   }
   const float* ct = (is_v ? cos_v : cos_qk) + static_cast<int64_t>(p) * half;
   const float* st = (is_v ? sin_v : sin_qk) + static_cast<int64_t>(p) * half;
@@ -74,14 +77,14 @@ __global__ void __launch_bounds__(256) turn_norm_write_kernel(T* __restrict__ qk
   for (int n = 0; n < kPairs; ++n) {
     const int i = lane + n * kWave;
     if (i < half) {
-      store_f32(dst + i, static_cast<float>(static_cast<Acc>(a[n]) * inv));
-      store_f32(dst + i + half, static_cast<float>(static_cast<Acc>(b[n]) * inv));
+      store_f32(dst + i * step, static_cast<float>(static_cast<Acc>(a[n]) * inv));
+      store_f32(dst + (i + half) * step, static_cast<float>(static_cast<Acc>(b[n]) * inv));
     }
   }
 #pragma unroll
   for (int n = 0; n < kPass; ++n) {
     const int c = 2 * half + lane + n * kWave;
-    if (c < width) store_f32(dst + c, static_cast<float>(static_cast<Acc>(rest[n]) * inv));
+    if (c < width) store_f32(dst + c * step, static_cast<float>(static_cast<Acc>(rest[n]) * inv));
   }
 }
 
@@ -175,13 +178,13 @@ __global__ void __launch_bounds__(256) talking_attention_kernel(
     for (int jj = 0; jj < n_keys; ++jj) {
       const int j = j0 + jj;
       const int64_t blk = table[j / block_size];
-      const T* vrow = v_cache + ((blk * kv_heads) * block_size + (j % block_size)) * static_cast<int64_t>(dv);
+      const T* vrow = v_cache + blk * kv_heads * static_cast<int64_t>(dv) * block_size + (j % block_size);
 #pragma unroll
       for (int n = 0; n < kTalkOwn; ++n) {
         const int e = tid + n * 256;
         if (e < outputs) {
           const int h = e / dv, c = e % dv;
-          acc[n] += static_cast<Acc>(Wm[h * kWave + jj]) * static_cast<Acc>(load_f32(vrow + static_cast<int64_t>(h / per) * block_size * dv + c));
+          acc[n] += static_cast<Acc>(Wm[h * kWave + jj]) * static_cast<Acc>(load_f32(vrow + (static_cast<int64_t>(h / per) * dv + c) * block_size));
         }
       }
     }
@@ -212,9 +215,58 @@ __global__ void __launch_bounds__(256) talking_attention_kernel(
   }
 }
 
+// ---- the heads' talk after the fact ---------------------------------------------------------------------
+// Mixing the heads' weights is linear in what the weights are applied to: with A[c][g] = sum_j p_g(j) v_c(j), the
+// unmixed weights of query head g applied to the values of value head c (float rows [kv_heads][T][heads * dv], from
+// the matrix-core attention kernels run once per value head), head h's result is sum_g M[h, g] A[c(h)][g]. A thread owns
+// a pair of channels (i, i + dv/2) of one head: sums over g in ascending order, turns the pair back by the row's
+// position and multiplies by the sigmoid of the gate.
+template <typename T>
+__global__ void __launch_bounds__(256) talk_mix_kernel(T* __restrict__ out, int64_t out_stride, const float* __restrict__ applied, int64_t plane,
+                                                       const int32_t* __restrict__ positions, int heads, int kv_heads, int dv,
+                                                       const float* __restrict__ talk, const float* __restrict__ cos_v, const float* __restrict__ sin_v,
+                                                       const T* __restrict__ gate, int64_t gate_stride) {
+  const int t = blockIdx.x, half = dv / 2, per = heads / kv_heads;
+  for (int e = threadIdx.x; e < heads * half; e += 256) {
+    const int h = e / half, i = e % half;
+    const float* src = applied + static_cast<int64_t>(h / per) * plane + static_cast<int64_t>(t) * heads * dv + i;
+    float x0 = 0.f, x1 = 0.f;
+    for (int g = 0; g < heads; ++g) {
+      const float w = talk ? talk[h * heads + g] : (g == h ? 1.f : 0.f);
+      x0 += w * src[g * dv];
+      x1 += w * src[g * dv + half];
+    }
+    float y0 = x0, y1 = x1;
+    if (cos_v) {
+      const int p = positions[t];
+      const float cs = cos_v[static_cast<int64_t>(p) * half + i], sn = sin_v[static_cast<int64_t>(p) * half + i];
+      y0 = x0 * cs + x1 * sn;
+      y1 = x1 * cs - x0 * sn;
+    }
+    const int64_t at = static_cast<int64_t>(h) * dv + i;
+    if (gate) {
+      y0 = y0 / (1.f + expf(-load_f32(gate + static_cast<int64_t>(t) * gate_stride + at)));
+      y1 = y1 / (1.f + expf(-load_f32(gate + static_cast<int64_t>(t) * gate_stride + at + half)));
+    }
+    store_f32(out + static_cast<int64_t>(t) * out_stride + at, y0);
+    store_f32(out + static_cast<int64_t>(t) * out_stride + at + half, y1);
+  }
+}
+
 }  // namespace alofa
 
 using namespace alofa;
+
+extern "C" int alofa_talk_mix(void* out, int64_t out_stride, int dtype, const float* applied, const int32_t* positions, int tokens, int heads, int kv_heads, int dv,
+                              const float* talk, const float* cos_v, const float* sin_v, const void* gate, int64_t gate_stride, hipStream_t stream) {
+  ALOFA_REQUIRE(tokens >= 0 && heads > 0 && kv_heads > 0 && heads % kv_heads == 0 && dv > 0 && dv % 2 == 0, "talk_mix: tokens=%d heads=%d kv_heads=%d dv=%d (kv_heads divides heads; an even value size)", tokens, heads, kv_heads, dv);
+  ALOFA_REQUIRE(!cos_v || (sin_v && positions), "talk_mix: turning back needs cos, sin and positions");
+  if (tokens == 0) return 0;
+  const int64_t plane = static_cast<int64_t>(tokens) * heads * dv;
+  if (dtype == kF32) talk_mix_kernel<float><<<tokens, 256, 0, stream>>>(static_cast<float*>(out), out_stride, applied, plane, positions, heads, kv_heads, dv, talk, cos_v, sin_v, static_cast<const float*>(gate), gate_stride);
+  else talk_mix_kernel<bf16_t><<<tokens, 256, 0, stream>>>(static_cast<bf16_t*>(out), out_stride, applied, plane, positions, heads, kv_heads, dv, talk, cos_v, sin_v, static_cast<const bf16_t*>(gate), gate_stride);
+  return check_launch("talk_mix");
+}
 
 extern "C" int alofa_turn_norm_write(void* qkv, int64_t stride, int dtype, const int32_t* positions, const float* cos_qk, const float* sin_qk, int half_qk,
                                      const float* cos_v, const float* sin_v, const int64_t* slots, void* k_cache, void* v_cache, int block_size,

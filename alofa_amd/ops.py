@@ -634,7 +634,8 @@ def paged_attention(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, v
 
 
 def _attention_operands(out, q, k_cache, v_cache, block_table, heads, kv_heads, d):
-    _gpu("out", out, torch.bfloat16, 2), _gpu("q", q, torch.bfloat16, 2)
+    # (float32 ``out``: the kernels leave their results unrounded there)
+    _gpu("out", out, torch.float32 if out.dtype is torch.float32 else torch.bfloat16, 2), _gpu("q", q, torch.bfloat16, 2)
     T = q.shape[0]
     if out.shape[0] != T or out.shape[1] < heads * d or q.shape[1] < heads * d:
         raise AlofaError("shape_mismatch", "attention rows do not fit", f"out={tuple(out.shape)} q={tuple(q.shape)} heads={heads} d={d}")
@@ -646,14 +647,15 @@ def _attention_operands(out, q, k_cache, v_cache, block_table, heads, kv_heads, 
     if bs < MIN_FAST_PAGE or bs & (bs - 1):
         raise AlofaError("unsupported", f"the bfloat16 attention kernels take pages of a power of two of tokens, at least {MIN_FAST_PAGE}", f"block_size={bs}")
     _gpu("block_table", block_table, torch.int32, 2), _contig("block_table", block_table)
-    if _rows("q", q) % 8 or q.data_ptr() % 16 or _rows("out", out) % 4 or out.data_ptr() % 8:
+    if _rows("q", q) % 8 or q.data_ptr() % 16 or _rows("out", out) % 4 or out.data_ptr() % (16 if out.dtype is torch.float32 else 8):
         raise AlofaError("alignment", "attention rows must be 16-byte aligned", f"q_stride={_rows('q', q)} out_stride={_rows('out', out)}")
     return T, bs
 
 
 def attention_decode(out, q, k_cache, v_cache, block_table, req_of_token, positions, heads, kv_heads, d, window, scale,
                      max_context: int, scratch: Optional[torch.Tensor], rows: Optional[torch.Tensor] = None,
-                     rope: Optional[tuple] = None, n_splits: Optional[int] = None, hand_over: Optional[bool] = None) -> None:
+                     rope: Optional[tuple] = None, n_splits: Optional[int] = None, hand_over: Optional[bool] = None,
+                     v_head: Optional[int] = None) -> None:
     """bfloat16 attention for tokens of requests that bring few tokens: every
     token of the batch, or the tokens ``rows`` (int32 indices into the batch).
     ``req_of_token`` None: every request brings one token and token i is request
@@ -664,7 +666,9 @@ def attention_decode(out, q, k_cache, v_cache, block_table, req_of_token, positi
     registers and writes them to the token's cache slot (``can_fuse_rope_into_decode``).
     ``n_splits`` (default ``decode_splits``): blocks that share the keys of a (token, key head);
     ``hand_over`` (default ``decode_hand_over``): the last of them to arrive combines their states,
-    else the states go to ``scratch`` and a second kernel combines them."""
+    else the states go to ``scratch`` and a second kernel combines them.
+    ``v_head``: every query head's weights meet the values of this one value head (the keys stay its own key head's).
+    ``out`` may be float32: the results are then stored unrounded."""
     T, bs = _attention_operands(out, q, k_cache, v_cache, block_table, heads, kv_heads, d)
     for n, t in (("req_of_token", req_of_token), ("positions", positions)):
         if t is None and n == "req_of_token":
@@ -702,10 +706,13 @@ def attention_decode(out, q, k_cache, v_cache, block_table, req_of_token, positi
     floats = n_tok * heads * n_splits * (d + 2) if n_splits > 1 and not hand_over else 0
     if floats and (scratch is None or scratch.dtype is not torch.float32 or not scratch.is_cuda or scratch.numel() < floats or not scratch.is_contiguous()):
         raise AlofaError("invalid_argument", "decode attention needs a float32 scratch buffer", f"floats={floats}")
-    _call("alofa_attention_decode", _ptr(out), _L(_rows("out", out)), _ptr(scratch if floats else None), _ptr(q), _L(_rows("q", q)),
+    if v_head is not None and (rope is not None or not 0 <= v_head < kv_heads):
+        raise AlofaError("invalid_argument", "a value head of its own: one of the value heads, and not with the rotary variant", f"v_head={v_head} kv_heads={kv_heads}")
+    as32 = out.dtype is torch.float32
+    _call("alofa_attention_decode_v", _ptr(None if as32 else out), _L(_rows("out", out)), _ptr(scratch if floats else None), _ptr(q), _L(_rows("q", q)),
           _ptr(k_cache), _ptr(v_cache), _ptr(block_table), _I(block_table.shape[1]), _ptr(req_of_token), _ptr(positions), _ptr(rows),
           _I(n_tok), _I(heads), _I(kv_heads), _I(d), _I(bs), _I(int(window or 0)), _F(scale), _I(n_splits),
-          _ptr(cos), _ptr(sin), _ptr(slots), _I(int(hand_over)), _stream())
+          _ptr(cos), _ptr(sin), _ptr(slots), _I(int(hand_over)), _I(-1 if v_head is None else v_head), _ptr(out if as32 else None), _stream())
 
 
 def can_fuse_rope_into_decode(d: int) -> bool:
@@ -780,22 +787,26 @@ def pair_tiles(runs: list, window: Optional[int] = None, heads: Optional[int] = 
 
 
 def attention_prefill(out, q, k_cache, v_cache, block_table, tiles, heads, kv_heads, d, window, scale, share: int = 0,
-                      rows: int = 16) -> None:
+                      rows: int = 16, v_head: Optional[int] = None) -> None:
     """bfloat16 attention for portions of prompts. ``tiles`` is int32 [n, 2, 4]
     from ``pair_tiles``: per block up to two runs of rows, each (request index,
     first row, rows <= 64 or 0 for none, position of the first row). ``share``
     (from ``prefill_share``; the tiles were paired for its count of blocks):
     that many heads of a group are served from one staged tile. ``rows``: query rows a wave owns
-    (from ``prefill_rows``; the tiles were paired for it too)."""
+    (from ``prefill_rows``; the tiles were paired for it too). ``v_head``: every query head's weights meet the values of this one
+    value head. ``out`` may be float32: the results are then stored unrounded."""
     T, bs = _attention_operands(out, q, k_cache, v_cache, block_table, heads, kv_heads, d)
     if d not in PREFILL_HEAD_DIMS:
         raise AlofaError("unsupported", "the prefill attention kernel is not built for this head size", f"head_dim={d} built={PREFILL_HEAD_DIMS}")
     _gpu("tiles", tiles, torch.int32, 3), _contig("tiles", tiles)
     if tuple(tiles.shape[1:]) != (2, 4) or tiles.shape[0] == 0:
         raise AlofaError("shape_mismatch", "tiles must be [n, 2, 4]", f"tiles={tuple(tiles.shape)}")
-    _call("alofa_attention_prefill", _ptr(out), _L(_rows("out", out)), _ptr(q), _L(_rows("q", q)), _ptr(k_cache), _ptr(v_cache),
+    if v_head is not None and not 0 <= v_head < kv_heads:
+        raise AlofaError("invalid_argument", "a value head of its own: one of the value heads", f"v_head={v_head} kv_heads={kv_heads}")
+    as32 = out.dtype is torch.float32
+    _call("alofa_attention_prefill_v", _ptr(None if as32 else out), _L(_rows("out", out)), _ptr(q), _L(_rows("q", q)), _ptr(k_cache), _ptr(v_cache),
           _ptr(block_table), _I(block_table.shape[1]), _ptr(tiles), _I(tiles.shape[0]), _I(heads), _I(kv_heads), _I(d), _I(bs),
-          _I(int(window or 0)), _F(scale), _I(share), _I(rows), _stream())
+          _I(int(window or 0)), _F(scale), _I(share), _I(rows), _I(-1 if v_head is None else v_head), _ptr(out if as32 else None), _stream())
 
 
 # ------------------------------------------------------------------ sampling
@@ -811,7 +822,7 @@ def turn_norm_write(qkv: torch.Tensor, positions: torch.Tensor, qk_table: tuple,
     heads, value heads side by side (``kv_heads`` 0: queries only). Queries and keys are turned on their first channels by ``qk_table``
     (cos, sin float32 [n, pairs]: channel i with i + pairs) and, with ``unit_norm``, divided by their root mean square over d; values are
     turned on all channels by ``v_table`` [n, dv / 2]. Queries are left in place; keys go to ``k_cache`` [pages, kv_heads, page, d] and
-    values to ``v_cache`` [pages, kv_heads, page, dv] at ``slots`` int64 [T]."""
+    values, transposed, to ``v_cache`` [pages, kv_heads, dv, page] at ``slots`` int64 [T]."""
     _gpu("qkv", qkv, None, 2), _gpu("positions", positions, torch.int32, 1), _contig("positions", positions)
     T = qkv.shape[0]
     cos, sin = qk_table
@@ -828,7 +839,7 @@ def turn_norm_write(qkv: torch.Tensor, positions: torch.Tensor, qk_table: tuple,
         _contig("k_cache", k_cache), _contig("v_cache", v_cache)
         block = k_cache.shape[2]
         if (cv.shape[1] != dv // 2 or cv.shape != sv.shape or cv.shape[0] < cos.shape[0] or slots.shape[0] != T or tuple(k_cache.shape[1:]) != (kv_heads, block, d)
-                or tuple(v_cache.shape) != (k_cache.shape[0], kv_heads, block, dv)):
+                or tuple(v_cache.shape) != (k_cache.shape[0], kv_heads, dv, block)):
             raise AlofaError("shape_mismatch", "caches, slots or the values' table do not fit", f"k={tuple(k_cache.shape)} v={tuple(v_cache.shape)} table={tuple(cv.shape)} slots={tuple(slots.shape)}")
     _call("alofa_turn_norm_write", _ptr(qkv), _L(_rows("qkv", qkv)), _I(dtype_code(qkv)), _ptr(positions), _ptr(cos), _ptr(sin), _I(half), _ptr(cv), _ptr(sv),
           _ptr(slots), _ptr(k_cache), _ptr(v_cache), _I(block), _I(T), _I(heads), _I(kv_heads), _I(d), _I(dv), _F(eps), _I(int(unit_norm)), _I(int(exact)), _stream())
@@ -839,14 +850,14 @@ def talking_attention(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor,
                       scale: float, talk: Optional[torch.Tensor], v_table: Optional[tuple], gate: Optional[torch.Tensor], exact: bool = False) -> None:
     """out[t, h] = turn_back(sum_j (sum_g talk[h, g] softmax_g(t, j)) v[j, h // group]) * sigmoid(gate[t, h]): softmax per query head g over
     the keys row t may see (its request's, up to its position; the last ``window`` of them), weights mixed over heads by ``talk`` [heads,
-    heads] (None: not mixed), values [pages, kv_heads, page, dv] that were turned by their positions (``v_table``: the result is turned back
+    heads] (None: not mixed), values [pages, kv_heads, dv, page] that were turned by their positions (``v_table``: the result is turned back
     by the row's; None: nothing is turned). ``q`` [T, heads * d] and ``out``, ``gate`` [T, heads * dv] rows (row strides allowed)."""
     _gpu("out", out, None, 2), _gpu("q", q, out.dtype, 2), _gpu("k_cache", k_cache, out.dtype, 4), _gpu("v_cache", v_cache, out.dtype, 4)
     _contig("k_cache", k_cache), _contig("v_cache", v_cache), _gpu("block_table", block_table, torch.int32, 2), _contig("block_table", block_table)
     _gpu("positions", positions, torch.int32, 1), _contig("positions", positions)
     T, block = q.shape[0], k_cache.shape[2]
     if (tuple(q.shape) != (T, heads * d) or tuple(out.shape) != (T, heads * dv) or tuple(k_cache.shape[1:]) != (kv_heads, block, d)
-            or tuple(v_cache.shape) != (k_cache.shape[0], kv_heads, block, dv) or positions.shape[0] != T):
+            or tuple(v_cache.shape) != (k_cache.shape[0], kv_heads, dv, block) or positions.shape[0] != T):
         raise AlofaError("shape_mismatch", "attention operands do not fit", f"out={tuple(out.shape)} q={tuple(q.shape)} k={tuple(k_cache.shape)} v={tuple(v_cache.shape)} heads={heads} kv_heads={kv_heads} d={d} dv={dv}")
     if req_of_token is not None:
         _gpu("req_of_token", req_of_token, torch.int32, 1), _contig("req_of_token", req_of_token)
@@ -869,6 +880,34 @@ def talking_attention(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor,
     _call("alofa_talking_attention", _ptr(out), _L(_rows("out", out)), _ptr(q), _L(_rows("q", q)), _ptr(k_cache), _ptr(v_cache), _I(dtype_code(out)),
           _ptr(block_table), _I(block_table.shape[1]), _ptr(req_of_token), _ptr(positions), _I(T), _I(heads), _I(kv_heads), _I(d), _I(dv), _I(block),
           _I(int(window or 0)), _F(scale), _ptr(talk), _ptr(cv), _ptr(sv), _ptr(gate), _L(_rows("gate", gate) if gate is not None else 0), _I(int(exact)), _stream())
+
+
+def talk_mix(out: torch.Tensor, applied: torch.Tensor, positions: torch.Tensor, heads: int, kv_heads: int, dv: int, talk: Optional[torch.Tensor],
+             v_table: Optional[tuple], gate: Optional[torch.Tensor]) -> None:
+    """The heads' talk after the fact: ``applied`` float32 [kv_heads, T, heads * dv] holds, per value head c, every query head's unmixed
+    softmax weights applied to the values of c; out[t, h] = turn_back(sum_g talk[h, g] applied[h // group, t, g]) * sigmoid(gate[t, h])
+    (``talk`` None: head h alone; ``v_table`` None: nothing is turned; ``gate`` None: no gate)."""
+    _gpu("out", out, None, 2), _gpu("applied", applied, torch.float32, 3), _contig("applied", applied)
+    _gpu("positions", positions, torch.int32, 1), _contig("positions", positions)
+    T = out.shape[0]
+    if tuple(applied.shape) != (kv_heads, T, heads * dv) or out.shape[1] != heads * dv or positions.shape[0] != T or heads % kv_heads or dv % 2:
+        raise AlofaError("shape_mismatch", "the applied weights do not fit", f"applied={tuple(applied.shape)} out={tuple(out.shape)} heads={heads} kv_heads={kv_heads} dv={dv}")
+    if talk is not None:
+        _gpu("talk", talk, torch.float32, 2), _contig("talk", talk)
+        if tuple(talk.shape) != (heads, heads):
+            raise AlofaError("shape_mismatch", "the heads' mixing matrix is [heads, heads]", f"talk={tuple(talk.shape)}")
+    cv = sv = None
+    if v_table is not None:
+        cv, sv = v_table
+        _gpu("cos_v", cv, torch.float32, 2), _gpu("sin_v", sv, torch.float32, 2), _contig("cos_v", cv), _contig("sin_v", sv)
+        if cv.shape[1] != dv // 2 or cv.shape != sv.shape:
+            raise AlofaError("shape_mismatch", "the values' table does not fit", f"table={tuple(cv.shape)} dv={dv}")
+    if gate is not None:
+        _gpu("gate", gate, out.dtype, 2)
+        if gate.shape != out.shape:
+            raise AlofaError("shape_mismatch", "one gate per output", f"gate={tuple(gate.shape)} out={tuple(out.shape)}")
+    _call("alofa_talk_mix", _ptr(out), _L(_rows("out", out)), _I(dtype_code(out)), _ptr(applied), _ptr(positions), _I(T), _I(heads), _I(kv_heads), _I(dv),
+          _ptr(talk), _ptr(cv), _ptr(sv), _ptr(gate), _L(_rows("gate", gate) if gate is not None else 0), _stream())
 
 
 def _store_operands(store, store_index, n: int):

@@ -10,8 +10,14 @@ sigmoid(Wg x) (``gate``), and projected by Wo.
 A layer may have no key and value projections of its own and read the pages of an earlier layer (``owns_cache`` False; its run entry
 names that layer with ``cache_of``): it brings its own queries, window, mixing matrix and gate.
 
-The pages hold keys as [kv_head, slot, head_dim] and values as [kv_head, slot, v_head_dim] (``keep_window``: how long they are kept:
-the longest window among the layers that read them)."""
+The pages hold keys as [kv_head, slot, head_dim] and values transposed, [kv_head, v_head_dim, slot], as the other attention parts'
+(``keep_window``: how long they are kept: the longest window among the layers that read them).
+
+Mixing the weights is linear in what they are applied to: head h's result is sum_g M[h, g] A[c(h)][g], where A[c][g] are query head g's
+unmixed weights applied to the values of value head c. In bfloat16, with pages of a power of two and heads of one size that the
+matrix-core attention kernels are built for, those kernels run once per value head (portions of prompts through the prefill kernel,
+single tokens through the decode kernel, as in ``paged_attend``) and leave A unrounded; one small kernel then mixes, turns back and
+gates. Every other case (float32, other sizes) runs the always-valid kernel, a block per row."""
 from __future__ import annotations
 
 import torch
@@ -19,6 +25,7 @@ import torch
 from .. import ops
 from ..errors import AlofaError
 from ..weights.loader import TensorRule
+from .attention import RowPlan
 from .base import SLOT, CacheNeed, CacheTensor, Mixer, build_part, register_part
 
 NAMES = {"q": "q", "k": "k", "v": "v", "o": "o", "gate": "g", "talk": "talk"}
@@ -81,12 +88,38 @@ class TalkingAttention(Mixer):
         self.qkv_width = self.q_width + (self.kv_heads * (self.d + self.dv) if self.owns else 0)
 
     def cache_need(self):
-        return CacheNeed((CacheTensor("k", (self.kv_heads, SLOT, self.d)), CacheTensor("v", (self.kv_heads, SLOT, self.dv))), self.keep_window)
+        return CacheNeed((CacheTensor("k", (self.kv_heads, SLOT, self.d)), CacheTensor("v", (self.kv_heads, self.dv, SLOT))), self.keep_window)
 
     def prepare(self, n_positions):
         self.position.table(n_positions)
         if self.value_position is not None:
             self.value_position.table(n_positions)
+
+    def _on_matrix_cores(self, ctx, kc, proj) -> bool:
+        page = kc.shape[2]
+        plan = ctx.memo("gqa_attention.rows", lambda: RowPlan(ctx))
+        return (not self.rt.exact and self.rt.dtype is torch.bfloat16 and self.d == self.dv and self.d % 16 == 0
+                and page >= ops.MIN_FAST_PAGE and page & (page - 1) == 0 and proj.stride(0) % 8 == 0 and (self.heads * self.dv) % 4 == 0
+                and (plan.long_runs is None or self.d in ops.PREFILL_HEAD_DIMS))
+
+    def _attend_per_value_head(self, ctx, q, kc, vc, table, attn, v_table, gate) -> None:
+        T = q.shape[0]
+        plan = ctx.memo("gqa_attention.rows", lambda: RowPlan(ctx))
+        applied = ctx.scratch("talking_applied", (self.kv_heads, T, self.heads * self.dv), torch.float32)
+        common = (self.heads, self.kv_heads, self.d, self.window, self.scale)
+        partial = None
+        if plan.n_short:
+            floats = ops.decode_scratch_floats(plan.n_short, self.heads, self.kv_heads, self.d, ctx.max_context, self.window)
+            partial = ctx.scratch("attn_partial", (floats,), torch.float32) if floats else None
+        one_each = ctx.max_q_len == 1 and plan.short_rows is None and plan.long_runs is None
+        for c in range(self.kv_heads):
+            if plan.long_runs is not None:
+                tiles, share, rows = plan.tiles(self.heads, self.kv_heads, self.d, self.window)
+                ops.attention_prefill(applied[c], q, kc, vc, table, tiles, *common, share=share, rows=rows, v_head=c)
+            if plan.n_short:
+                ops.attention_decode(applied[c], q, kc, vc, table, None if one_each else ctx.req_of_token, ctx.positions, *common,
+                                     ctx.max_context, partial, rows=plan.short_rows, v_head=c)
+        ops.talk_mix(attn, applied, ctx.positions, self.heads, self.kv_heads, self.dv, self.talk, v_table, gate)
 
     def forward(self, ctx, where, x, residual, out=None):
         T, exact = residual.shape[0], self.rt.exact
@@ -101,8 +134,12 @@ class TalkingAttention(Mixer):
                             self.kv_heads if self.owns else 0, self.d, self.dv, self.eps, self.unit_norm, exact,
                             kv.slots if self.owns else None, kc if self.owns else None, vc if self.owns else None)
         attn = ctx.scratch("talking_out", (T, self.heads * self.dv), self.rt.dtype)
-        ops.talking_attention(attn, proj[:, :self.q_width], kc, vc, kv.block_table, ctx.req_of_token, ctx.positions, self.heads, self.kv_heads,
-                              self.d, self.dv, self.window, self.scale, self.talk, v_table, proj[:, self.gate_at:] if self.gated else None, exact)
+        gate = proj[:, self.gate_at:] if self.gated else None
+        if self._on_matrix_cores(ctx, kc, proj):
+            self._attend_per_value_head(ctx, proj[:, :self.q_width], kc, vc, kv.block_table, attn, v_table, gate)
+        else:
+            ops.talking_attention(attn, proj[:, :self.q_width], kc, vc, kv.block_table, ctx.req_of_token, ctx.positions, self.heads, self.kv_heads,
+                                  self.d, self.dv, self.window, self.scale, self.talk, v_table, gate, exact)
         if out is not None:
             ops.gemm(out, attn, self.w_o, exact=exact)
         else:

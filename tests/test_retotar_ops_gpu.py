@@ -22,10 +22,13 @@ def tables(base, n, positions, factor=1.0):
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("H,G,d,dv,dims,window", [(4, 2, 16, 24, 8, 20), (3, 1, 24, 40, 24, 7), (2, 2, 32, 16, 2, None), (8, 4, 64, 32, 32, 33),
-                                                  (5, 5, 10, 6, 4, 16), (12, 3, 128, 128, 64, 48), (6, 6, 9, 2, 6, 1)])
+                                                  (5, 5, 10, 6, 4, 16), (12, 3, 128, 128, 64, 48), (6, 6, 9, 2, 6, 1), (4, 2, 32, 32, 16, 20),
+                                                  (6, 6, 16, 16, 8, None), (8, 2, 64, 64, 32, 33), (16, 1, 48, 48, 48, 5)])
 def test_attention_over_shuffled_pages_in_portions(H, G, d, dv, dims, window, dtype):
     """Three requests of unequal length whose rows come in portions, mixed in every call; queries and keys turned and normed, values
-    turned and the result turned back, the heads' weights mixed, the gate: against the plain functions on the whole sequences."""
+    turned and the result turned back, the heads' weights mixed, the gate: against the plain functions on the whole sequences. Where
+    the matrix-core kernels take the sizes (bfloat16, heads of one size in steps of 16), the same rows also go through them, once per
+    value head, and through the kernel that mixes afterwards."""
     from alofa_amd import ops
     g = torch.Generator().manual_seed(H * 100 + d)
     exact = dtype is torch.float32
@@ -38,7 +41,7 @@ def test_attention_over_shuffled_pages_in_portions(H, G, d, dv, dims, window, dt
         for b in range((n + page - 1) // page):
             table[r, b] = order.pop()
     kc = torch.zeros(n_pages, G, page, d, dtype=dtype, device=DEV)
-    vc = torch.zeros(n_pages, G, page, dv, dtype=dtype, device=DEV)
+    vc = torch.zeros(n_pages, G, dv, page, dtype=dtype, device=DEV)
     talk = torch.eye(H, dtype=F) + 0.3 * torch.randn(H, H, generator=g, dtype=F)
     qk_t, v_t = tables(base, dims, 128, factor), tables(base, dv, 128)
     width = H * d + G * (d + dv)
@@ -60,6 +63,8 @@ def test_attention_over_shuffled_pages_in_portions(H, G, d, dv, dims, window, dt
         want.append(o.reshape(n, H * dv) * torch.sigmoid(x[:, width:]))
     # the kernels, in calls that mix portions of the three requests
     got = [torch.zeros(n, H * dv, dtype=F) for n in lengths]
+    fast = not exact and d == dv and d % 16 == 0
+    got_fast = [torch.zeros(n, H * dv, dtype=F) for n in lengths]
     done = [0, 0, 0]
     plans = [cuts(70, (31, 2, 1, 17)), cuts(33, (2, 9, 1, 1)), cuts(51, (16, 1, 20, 3))]
     for step in range(max(len(p) for p in plans)):
@@ -71,15 +76,38 @@ def test_attention_over_shuffled_pages_in_portions(H, G, d, dv, dims, window, dt
         ops.turn_norm_write(rows[:, :width], positions, qk_t, v_t, H, G, d, dv, eps, True, exact, slots, kc, vc)
         out = torch.empty(rows.shape[0], H * dv, dtype=dtype, device=DEV)
         ops.talking_attention(out, rows[:, :H * d], kc, vc, table.to(DEV), req, positions, H, G, d, dv, window, scale, dev(talk.numpy()), v_t, rows[:, width:], exact)
+        if fast:
+            # portions of more than a few rows through the prefill kernel in runs of up to 64, the others row by row through the decode kernel
+            runs, short, row = [], [], 0
+            for r, a, b in live:
+                if b - a > ops.DECODE_MAX_Q:
+                    runs += [(r, row + q0, min(64, b - a - q0), a + q0) for q0 in range(0, b - a, 64)]
+                else:
+                    short += list(range(row, row + b - a))
+                row += b - a
+            applied = torch.full((G, rows.shape[0], H * dv), float("nan"), device=DEV)
+            for c in range(G):
+                if runs:
+                    tiles = torch.tensor(ops.pair_tiles(runs, window, H), dtype=torch.int32, device=DEV)
+                    ops.attention_prefill(applied[c], rows[:, :H * d], kc, vc, table.to(DEV), tiles, H, G, d, window, scale, v_head=c)
+                if short:
+                    floats = ops.decode_scratch_floats(len(short), H, G, d, 128, window)
+                    ops.attention_decode(applied[c], rows[:, :H * d], kc, vc, table.to(DEV), req, positions, H, G, d, window, scale, 128,
+                                         torch.empty(max(floats, 1), device=DEV), rows=torch.tensor(short, dtype=torch.int32, device=DEV), v_head=c)
+            out_fast = torch.empty_like(out)
+            ops.talk_mix(out_fast, applied, positions, H, G, dv, dev(talk.numpy()), v_t, rows[:, width:])
         at = 0
         for r, a, b in live:
             got[r][a:b] = out[at:at + b - a].double().cpu()
+            if fast:
+                got_fast[r][a:b] = out_fast[at:at + b - a].double().cpu()
             at += b - a
             done[r] = b
     assert done == lengths
     for r in range(3):
-        err = (got[r] - want[r]).abs().max().item()
-        assert err <= (2e-5 if exact else 3e-2) * max(1.0, want[r].abs().max().item()), f"request {r}: {err}"
+        for which, rows_got in (("a block per row", got), ("matrix cores", got_fast)) if fast else (("a block per row", got),):
+            err = (rows_got[r] - want[r]).abs().max().item()
+            assert err <= (2e-5 if exact else 3e-2) * max(1.0, want[r].abs().max().item()), f"request {r} ({which}): {err}"
 
 
 @pytest.mark.parametrize("exact", [True, False])
