@@ -139,6 +139,63 @@ __global__ void __launch_bounds__(256) headnorm_gate_kernel(T* __restrict__ out,
   }
 }
 
+// The same for wide heads (several heads normed together as one row, say): a block of 256 threads per (token, head), the sum of squares over
+// the lanes of each wave and then over the four waves in their order.
+template <typename T, typename Acc>
+__global__ void __launch_bounds__(256) headnorm_gate_wide_kernel(T* __restrict__ out, int64_t out_stride, const float* __restrict__ o,
+                                                                 const T* __restrict__ g, int64_t g_stride, const float* __restrict__ w,
+                                                                 int tokens, int heads, int dv, float eps, float out_scale, int parts, int64_t part_stride,
+                                                                 int sigmoid_gate, int extra, const float* __restrict__ floor) {
+  __shared__ Acc wave_ss[4];
+  const int64_t unit = blockIdx.x;
+  const int t = static_cast<int>(unit / heads), h = static_cast<int>(unit % heads);
+  const float* src = o + (static_cast<int64_t>(t) * heads + h) * (dv + extra);
+  float under = 1.f;
+  if (floor) {
+    float n = 0.f;
+    for (int p = 0; p < parts; ++p) n += src[p * part_stride + dv];
+    under = fmaxf(fabsf(n), floor[static_cast<int64_t>(t) * heads + h]) + 1e-6f;
+  }
+  constexpr int kOwn = 8;      // values a thread keeps between the sum of squares and the scaling (rows up to 2,048 wide; wider ones are added again)
+  float own[kOwn];
+  Acc ss = 0;
+  auto value = [&](int j) {
+    float v = 0.f;
+    for (int p = 0; p < parts; ++p) v += src[p * part_stride + j];
+    return floor ? v / under : v;
+  };
+#pragma unroll
+  for (int c = 0; c < kOwn; ++c) {
+    const int j = threadIdx.x + c * 256;
+    own[c] = j < dv ? value(j) : 0.f;
+    ss += static_cast<Acc>(own[c]) * static_cast<Acc>(own[c]);
+  }
+  for (int j = threadIdx.x + kOwn * 256; j < dv; j += 256) {
+    const float v = value(j);
+    ss += static_cast<Acc>(v) * static_cast<Acc>(v);
+  }
+  ss = wave_sum(ss);
+  if (threadIdx.x % kWave == 0) wave_ss[threadIdx.x / kWave] = ss;
+  __syncthreads();
+  ss = ((wave_ss[0] + wave_ss[1]) + wave_ss[2]) + wave_ss[3];
+  const Acc inv = static_cast<Acc>(1) / sqrt(ss / static_cast<Acc>(dv) + static_cast<Acc>(eps));
+  const T* gate = g + static_cast<int64_t>(t) * g_stride + static_cast<int64_t>(h) * dv;
+  T* dst = out + static_cast<int64_t>(t) * out_stride + static_cast<int64_t>(h) * dv;
+  auto leave = [&](int j, float v) {
+    const Acc z = static_cast<Acc>(load_f32(gate + j));
+    const Acc silu = (sigmoid_gate ? static_cast<Acc>(1) : z) / (static_cast<Acc>(1) + exp(-z));
+    Acc y = static_cast<Acc>(v) * inv;
+    if (w) y *= static_cast<Acc>(w[h * dv + j]);
+    store_f32(dst + j, static_cast<float>(y * silu * static_cast<Acc>(out_scale)));
+  };
+#pragma unroll
+  for (int c = 0; c < kOwn; ++c) {
+    const int j = threadIdx.x + c * 256;
+    if (j < dv) leave(j, own[c]);
+  }
+  for (int j = threadIdx.x + kOwn * 256; j < dv; j += 256) leave(j, value(j));
+}
+
 // ---- activations -------------------------------------------------------------------------------
 // kind 0: xIELU with a = softplus(p) and b = 1/2 + softplus(q) given: z > 0: a z^2 + z/2; else b (exp(z) - 1 - z) + z/2.
 // kind 1: tanh. kind 2: silu, z sigmoid(z). In place or not; rows of `width` values with a row stride.
@@ -236,6 +293,13 @@ extern "C" int alofa_headnorm_gate(void* out, int64_t out_stride, const float* o
   ALOFA_REQUIRE(tokens >= 0 && heads > 0 && dv > 0 && eps > 0.f && parts >= 1, "headnorm_gate: bad sizes (tokens=%d heads=%d dv=%d)", tokens, heads, dv);
   ALOFA_REQUIRE(!exact || dtype == kF32, "headnorm_gate: the exact path is float32");
   if (tokens == 0) return 0;
+  if (dv > 256) {      // wide rows: a block each
+    const unsigned units = static_cast<unsigned>(static_cast<int64_t>(tokens) * heads);
+    if (exact) headnorm_gate_wide_kernel<float, double><<<units, 256, 0, stream>>>(static_cast<float*>(out), out_stride, o, static_cast<const float*>(g), g_stride, w, tokens, heads, dv, eps, out_scale, parts, part_stride, sigmoid_gate, extra, floor);
+    else if (dtype == kF32) headnorm_gate_wide_kernel<float, float><<<units, 256, 0, stream>>>(static_cast<float*>(out), out_stride, o, static_cast<const float*>(g), g_stride, w, tokens, heads, dv, eps, out_scale, parts, part_stride, sigmoid_gate, extra, floor);
+    else headnorm_gate_wide_kernel<bf16_t, float><<<units, 256, 0, stream>>>(static_cast<bf16_t*>(out), out_stride, o, static_cast<const bf16_t*>(g), g_stride, w, tokens, heads, dv, eps, out_scale, parts, part_stride, sigmoid_gate, extra, floor);
+    return check_launch("headnorm_gate");
+  }
   const unsigned grid = static_cast<unsigned>((static_cast<int64_t>(tokens) * heads + 3) / 4);
   if (exact) headnorm_gate_kernel<float, double><<<grid, 256, 0, stream>>>(static_cast<float*>(out), out_stride, o, static_cast<const float*>(g), g_stride, w, tokens, heads, dv, eps, out_scale, parts, part_stride, sigmoid_gate, extra, floor);
   else if (dtype == kF32) headnorm_gate_kernel<float, float><<<grid, 256, 0, stream>>>(static_cast<float*>(out), out_stride, o, static_cast<const float*>(g), g_stride, w, tokens, heads, dv, eps, out_scale, parts, part_stride, sigmoid_gate, extra, floor);

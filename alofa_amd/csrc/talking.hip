@@ -219,20 +219,36 @@ __global__ void __launch_bounds__(256) talking_attention_kernel(
 // Mixing the heads' weights is linear in what the weights are applied to: with A[c][g] = sum_j p_g(j) v_c(j), the
 // unmixed weights of query head g applied to the values of value head c (float rows [kv_heads][T][heads * dv], from
 // the matrix-core attention kernels run once per value head), head h's result is sum_g M[h, g] A[c(h)][g]. A thread owns
-// a pair of channels (i, i + dv/2) of one head: sums over g in ascending order, turns the pair back by the row's
+// a pair of channels (i, i + dv/2) of one head (a block per row and head): sums over g in ascending order, turns the pair back by the row's
 // position and multiplies by the sigmoid of the gate.
 template <typename T>
-__global__ void __launch_bounds__(256) talk_mix_kernel(T* __restrict__ out, int64_t out_stride, const float* __restrict__ applied, int64_t plane,
-                                                       const int32_t* __restrict__ positions, int heads, int kv_heads, int dv,
-                                                       const float* __restrict__ talk, const float* __restrict__ cos_v, const float* __restrict__ sin_v,
-                                                       const T* __restrict__ gate, int64_t gate_stride) {
-  const int t = blockIdx.x, half = dv / 2, per = heads / kv_heads;
-  for (int e = threadIdx.x; e < heads * half; e += 256) {
-    const int h = e / half, i = e % half;
-    const float* src = applied + static_cast<int64_t>(h / per) * plane + static_cast<int64_t>(t) * heads * dv + i;
+__global__ void __launch_bounds__(64) talk_mix_kernel(T* __restrict__ out, int64_t out_stride, const float* __restrict__ applied, int64_t plane,
+                                                      const int32_t* __restrict__ positions, int heads, int kv_heads, int dv,
+                                                      const float* __restrict__ talk, const float* __restrict__ cos_v, const float* __restrict__ sin_v,
+                                                      const T* __restrict__ gate, int64_t gate_stride) {
+  const int t = blockIdx.x, h = blockIdx.y, half = dv / 2, per = heads / kv_heads;
+  const float* rows = applied + static_cast<int64_t>(h / per) * plane + static_cast<int64_t>(t) * heads * dv;
+  const float* mix = talk ? talk + h * heads : nullptr;
+  for (int i = threadIdx.x; i < half; i += 64) {
+    const float* src = rows + i;
     float x0 = 0.f, x1 = 0.f;
-    for (int g = 0; g < heads; ++g) {
-      const float w = talk ? talk[h * heads + g] : (g == h ? 1.f : 0.f);
+    int g = 0;
+    for (; g + 4 <= heads; g += 4) {      // (four heads' loads on their way together; the sums in ascending order of g)
+      float a[4], b[4], w[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        a[u] = src[(g + u) * dv];
+        b[u] = src[(g + u) * dv + half];
+        w[u] = mix ? mix[g + u] : (g + u == h ? 1.f : 0.f);
+      }
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        x0 += w[u] * a[u];
+        x1 += w[u] * b[u];
+      }
+    }
+    for (; g < heads; ++g) {
+      const float w = mix ? mix[g] : (g == h ? 1.f : 0.f);
       x0 += w * src[g * dv];
       x1 += w * src[g * dv + half];
     }
@@ -263,8 +279,8 @@ extern "C" int alofa_talk_mix(void* out, int64_t out_stride, int dtype, const fl
   ALOFA_REQUIRE(!cos_v || (sin_v && positions), "talk_mix: turning back needs cos, sin and positions");
   if (tokens == 0) return 0;
   const int64_t plane = static_cast<int64_t>(tokens) * heads * dv;
-  if (dtype == kF32) talk_mix_kernel<float><<<tokens, 256, 0, stream>>>(static_cast<float*>(out), out_stride, applied, plane, positions, heads, kv_heads, dv, talk, cos_v, sin_v, static_cast<const float*>(gate), gate_stride);
-  else talk_mix_kernel<bf16_t><<<tokens, 256, 0, stream>>>(static_cast<bf16_t*>(out), out_stride, applied, plane, positions, heads, kv_heads, dv, talk, cos_v, sin_v, static_cast<const bf16_t*>(gate), gate_stride);
+  if (dtype == kF32) talk_mix_kernel<float><<<dim3(tokens, heads), 64, 0, stream>>>(static_cast<float*>(out), out_stride, applied, plane, positions, heads, kv_heads, dv, talk, cos_v, sin_v, static_cast<const float*>(gate), gate_stride);
+  else talk_mix_kernel<bf16_t><<<dim3(tokens, heads), 64, 0, stream>>>(static_cast<bf16_t*>(out), out_stride, applied, plane, positions, heads, kv_heads, dv, talk, cos_v, sin_v, static_cast<const bf16_t*>(gate), gate_stride);
   return check_launch("talk_mix");
 }
 

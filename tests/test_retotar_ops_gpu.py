@@ -139,7 +139,7 @@ def test_the_memory_with_gates_in_portions_of_two_requests(H, d, dv, dtype):
     exact, cap, eps = dtype is torch.float32, 7.0, 1e-5
     store = pt._id if exact else pt.to_bfloat16
     width = 2 * H * d + 2 * H * dv
-    lengths = [90, 41]
+    lengths = [290, 41]      # (portions of one row, of fewer and of more than a wavefront's 64 rows, and of exactly 128)
     raw = [store(torch.randn(n, width, generator=g, dtype=F)) for n in lengths]
     zs = [torch.randn(n, 2 * H, generator=g, dtype=torch.float32) * 3.0 for n in lengths]
     zs[0][:, H:] += 4.0      # (forget gates mostly open in one request, so that the maximum and the memory travel far)
@@ -152,7 +152,7 @@ def test_the_memory_with_gates_in_portions_of_two_requests(H, d, dv, dtype):
     want = [pt.mlstm(torch.cat([x, z.double()], 1), W, m, eps) for x, z in zip(raw, zs)]
     state, top = torch.zeros(3, H, d, dv + 1, device=DEV), torch.zeros(3, H, device=DEV)
     got = [torch.zeros(n, H * dv, dtype=F) for n in lengths]
-    plans = [cuts(90, (1, 33, 1, 2, 70)), cuts(41, (1, 7, 1, 30, 1))]
+    plans = [cuts(290, (1, 33, 1, 2, 70, 128, 64)), cuts(41, (1, 7, 1, 30, 1))]
     for step in range(max(len(p) for p in plans)):
         live = [(r, *plans[r][step]) for r in range(2) if step < len(plans[r])]
         rows = rows_of([(2 - r, b - a) for r, a, b in live], 3)
@@ -193,3 +193,20 @@ def test_the_norm_that_adds_and_the_row_handed_on():
             out, rows = dev(res), dev(x, dtype)
             ops.add_row_scaled(out, rows, dev(scale))
             assert (out.cpu().double() - (f32(res) + f32(scale)[:, None] * rows.cpu().double())).abs().max() <= 1e-5
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("heads,dv,parts", [(1, 300, 1), (1, 2048, 3), (2, 2500, 2), (3, 257, 1)])
+def test_wide_rows_normed_and_gated(heads, dv, parts, dtype):
+    """Heads wider than a wavefront's kernel takes (several heads normed together as one row): against the plain norm, weight and sigmoid gate."""
+    from alofa_amd import ops
+    g = torch.Generator().manual_seed(dv)
+    T, eps, exact = 5, 1e-5, dtype is torch.float32
+    o = torch.randn(parts + 1, T, heads * dv, generator=g, dtype=torch.float32)      # (one part more than is added: it must not be read)
+    gate = torch.randn(T, heads * dv, generator=g, dtype=torch.float32).to(dtype)
+    w = torch.randn(heads * dv, generator=g, dtype=torch.float32)
+    rows = o[:parts].double().sum(0).view(T, heads, dv)
+    want = (pt.unit_rms(rows, eps).reshape(T, heads * dv) * w.double()) * torch.sigmoid(gate.double())
+    out = torch.empty(T, heads * dv, dtype=dtype, device=DEV)
+    ops.headnorm_gate(out, o.to(DEV), gate.to(DEV), w.to(DEV), heads, dv, eps, exact, parts=parts, gate_kind="sigmoid")
+    assert (out.double().cpu() - want).abs().max() <= (2e-5 if exact else 3e-2) * max(1.0, want.abs().max().item())
