@@ -86,7 +86,8 @@ __device__ __forceinline__ Pair8 rotate8(uint4 lo, uint4 hi, float4 c_lo, float4
 }
 
 // DT = d / 16; NW: waves per block. blockIdx.y = key head * chunks + chunk of up to 16 heads of its group.
-template <int DT, int NW, bool kRope>
+// kSplit: a weight enters the second product as two bfloat16 numbers, its rounding and what the rounding took away: sixteen bits of every weight count.
+template <int DT, int NW, bool kRope, bool kSplit = false>
 __global__ void __launch_bounds__(64 * NW) attention_decode_kernel(
     bf16_t* __restrict__ out, int64_t out_stride, float* __restrict__ partial, const bf16_t* __restrict__ q,
     int64_t q_stride, bf16_t* __restrict__ k_cache, bf16_t* __restrict__ v_cache,
@@ -266,6 +267,11 @@ __global__ void __launch_bounds__(64 * NW) attention_decode_kernel(
     l = l * corr + sum;   // this lane's share of the head's sum; the four lanes of a head meet at the end
     const uint4 w = make_uint4(pack_bf16x2(pw[0], pw[1]), pack_bf16x2(pw[2], pw[3]), pack_bf16x2(pw[4], pw[5]), pack_bf16x2(pw[6], pw[7]));
     const bf16x8 pf = __builtin_bit_cast(bf16x8, w);
+    bf16x8 pl;
+    if constexpr (kSplit) {
+      const uint4 r = make_uint4(pack_bf16x2_rest(pw[0], pw[1], w.x), pack_bf16x2_rest(pw[2], pw[3], w.y), pack_bf16x2_rest(pw[4], pw[5], w.z), pack_bf16x2_rest(pw[6], pw[7], w.w));
+      pl = __builtin_bit_cast(bf16x8, r);
+    }
     // What lies beyond the visible keys is not data: it is cleared, so that a weight of zero times it is zero.
     // (Within lo..p a weight of zero meets a visible key's values.)
     uint32_t keep_x[2] = {0xffffffffu, 0xffffffffu}, keep_y[2] = {0xffffffffu, 0xffffffffu};
@@ -294,6 +300,7 @@ __global__ void __launch_bounds__(64 * NW) attention_decode_kernel(
       }
       const uint4 vv = make_uint4(vw[0], vw[1], vw[2], vw[3]);
       o[nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, vv), pf, o[nt], 0, 0, 0);
+      if constexpr (kSplit) o[nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, vv), pl, o[nt], 0, 0, 0);
     }
   };
 
@@ -547,7 +554,8 @@ extern "C" int alofa_attention_decode_v(void* out, int64_t out_stride, float* pa
                                         int max_blocks, const int32_t* req_of_token, const int32_t* positions,
                                         const int32_t* rows, int tokens, int heads, int kv_heads, int d, int block_size, int window,
                                         float scale, int n_splits, const float* cos_t, const float* sin_t, const int64_t* slots,
-                                        int hand_over, int v_head, float* out32, hipStream_t stream) {
+                                        int hand_over, int v_head, float* out32, int split, hipStream_t stream) {
+  ALOFA_REQUIRE(!split || !cos_t, "attention_decode: split weights and the rotary variant do not go together");
   ALOFA_REQUIRE(v_head < kv_heads && (v_head < 0 || !cos_t), "attention_decode: value head %d of %d (and none with the rotary variant)", v_head, kv_heads);
   ALOFA_REQUIRE(tokens > 0 && heads > 0 && kv_heads > 0 && heads % kv_heads == 0,
                 "attention_decode: tokens=%d heads=%d kv_heads=%d (kv_heads must divide heads)", tokens, heads, kv_heads);
@@ -574,7 +582,11 @@ extern "C" int alofa_attention_decode_v(void* out, int64_t out_stride, float* pa
   const RopeArgs rope{cos_t, sin_t, slots};
   dim3 grid(tokens, kv_heads * ((group + kHeadsPerBlock - 1) / kHeadsPerBlock), n_splits);
 #define ALOFA_DECODE(DT, NW, ROPE)                                                                                        \
-  attention_decode_kernel<DT, NW, ROPE><<<grid, 64 * NW, 0, stream>>>(                                                    \
+  if (split && !ROPE) attention_decode_kernel<DT, NW, false, true><<<grid, 64 * NW, 0, stream>>>(                         \
+      static_cast<bf16_t*>(out), out_stride, partial, static_cast<const bf16_t*>(q), q_stride,                            \
+      static_cast<bf16_t*>(k_cache), static_cast<bf16_t*>(v_cache), block_table, max_blocks, req_of_token,                \
+      positions, rows, heads, kv_heads, bs_shift, window, scale, rope, counters, v_head, out32);                          \
+  else attention_decode_kernel<DT, NW, ROPE><<<grid, 64 * NW, 0, stream>>>(                                                    \
       static_cast<bf16_t*>(out), out_stride, partial, static_cast<const bf16_t*>(q), q_stride,                            \
       static_cast<bf16_t*>(k_cache), static_cast<bf16_t*>(v_cache), block_table, max_blocks, req_of_token,                \
       positions, rows, heads, kv_heads, bs_shift, window, scale, rope, counters, v_head, out32)
@@ -622,5 +634,5 @@ extern "C" int alofa_attention_decode(void* out, int64_t out_stride, float* part
                                       float scale, int n_splits, const float* cos_t, const float* sin_t, const int64_t* slots,
                                       int hand_over, hipStream_t stream) {
   return alofa_attention_decode_v(out, out_stride, partial, q, q_stride, k_cache, v_cache, block_table, max_blocks, req_of_token, positions, rows, tokens,
-                                  heads, kv_heads, d, block_size, window, scale, n_splits, cos_t, sin_t, slots, hand_over, -1, nullptr, stream);
+                                  heads, kv_heads, d, block_size, window, scale, n_splits, cos_t, sin_t, slots, hand_over, -1, nullptr, 0, stream);
 }

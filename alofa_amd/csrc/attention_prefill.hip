@@ -60,7 +60,9 @@ constexpr int KPAD = 8, VPAD = 8;
 // (request index, first row in the packed batch, rows (<= 64; 0: none), position of the first row). The caller
 // pairs long runs with short ones so that blocks carry about the same number of key tiles.
 // kShare: blockIdx.y = key head * chunks + chunk of up to WPT query heads of its group; blockIdx.z = which RW rows of the run.
-template <int DT, int TEAMS, int WPT, bool kShare, int RW = 16, int KT = 64>  // DT = d / 16; RW: query rows per wave (16 or 32); KT: keys per tile (64; 32 with RW = 32)
+// kSplit: a weight enters the second product as two bfloat16 numbers, its rounding and what the rounding took away (two
+// matrix-core instructions per tile of values instead of one): sixteen bits of every weight count, for models whose weights are 32-bit by design.
+template <int DT, int TEAMS, int WPT, bool kShare, int RW = 16, int KT = 64, bool kSplit = false>  // DT = d / 16; RW: query rows per wave (16 or 32); KT: keys per tile (64; 32 with RW = 32)
 __global__ void __launch_bounds__(64 * WPT * TEAMS, (RW == 32 && 64 * WPT * TEAMS <= 256) ? 2 : 1) attention_prefill_kernel(
     bf16_t* __restrict__ out, int64_t out_stride, const bf16_t* __restrict__ q, int64_t q_stride,
     const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache, const int32_t* __restrict__ block_table,
@@ -73,6 +75,7 @@ __global__ void __launch_bounds__(64 * WPT * TEAMS, (RW == 32 && 64 * WPT * TEAM
   constexpr int OT = RW == 32 ? (d + 31) / 32 : DT;   // output tiles of 16 (RW = 32: of 32) channels
   constexpr int OV = RW == 32 ? 16 : 4;               // ... each this many values per lane
   static_assert(RW == 16 || RW == 32, "a wave owns 16 or 32 query rows");
+  static_assert(!kSplit || RW == 16, "split weights: in the 16-row form only");
   constexpr int KROW = d + KPAD, VROW = BKV + VPAD;
   // per team: its key tile and its transposed value tile; at the end the same room takes the team's
   // running state (per lane its maximum, its sum and its 4 * DT channels)
@@ -363,12 +366,17 @@ __global__ void __launch_bounds__(64 * WPT * TEAMS, (RW == 32 && 64 * WPT * TEAM
       }
     }
     l = l * corr + sum;   // this lane's share of the row's sum; the four lanes of a row meet at the end
-    bf16x8 pf[2];
+    bf16x8 pf[2], pl[2];
 #pragma unroll
     for (int half = 0; half < 2; ++half) {
       const uint4 w = make_uint4(pack_bf16x2(p[8 * half], p[8 * half + 1]), pack_bf16x2(p[8 * half + 2], p[8 * half + 3]),
                                  pack_bf16x2(p[8 * half + 4], p[8 * half + 5]), pack_bf16x2(p[8 * half + 6], p[8 * half + 7]));
       pf[half] = __builtin_bit_cast(bf16x8, w);
+      if constexpr (kSplit) {
+        const uint4 r = make_uint4(pack_bf16x2_rest(p[8 * half], p[8 * half + 1], w.x), pack_bf16x2_rest(p[8 * half + 2], p[8 * half + 3], w.y),
+                                   pack_bf16x2_rest(p[8 * half + 4], p[8 * half + 5], w.z), pack_bf16x2_rest(p[8 * half + 6], p[8 * half + 7], w.w));
+        pl[half] = __builtin_bit_cast(bf16x8, r);
+      }
     }
     // O^T += V^T P^T, one MFMA per 32-key half
 #pragma unroll
@@ -382,6 +390,7 @@ __global__ void __launch_bounds__(64 * WPT * TEAMS, (RW == 32 && 64 * WPT * TEAM
         const uint2 hi = *reinterpret_cast<const uint2*>(vrow + ((half * 32 + 16 + g * 4) ^ sw));
         const uint4 vv = make_uint4(lo.x, lo.y, hi.x, hi.y);
         o[nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, vv), pf[half], o[nt], 0, 0, 0);
+        if constexpr (kSplit) o[nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, vv), pl[half], o[nt], 0, 0, 0);
       }
     }
     }
@@ -504,10 +513,13 @@ extern "C" int alofa_attention_prefill_supports(int d) {
 
 // v_head >= 0: every query head's weights meet the values of that one value head (its keys stay its own key head's);
 // out32: the results go there unrounded, as float rows of `out`'s shape and stride (16-byte aligned), and `out` is not written.
+// split: the weights enter the second product with sixteen bits each (see kSplit).
 extern "C" int alofa_attention_prefill_v(void* out, int64_t out_stride, const void* q, int64_t q_stride,
                                          const void* k_cache, const void* v_cache, const int32_t* block_table,
                                          int max_blocks, const int32_t* tiles, int n_tiles, int heads, int kv_heads, int d,
-                                         int block_size, int window, float scale, int share, int rows_per_wave, int v_head, float* out32, hipStream_t stream) {
+                                         int block_size, int window, float scale, int share, int rows_per_wave, int v_head, float* out32, int split,
+                                         hipStream_t stream) {
+  ALOFA_REQUIRE(!split || (share == 0 && rows_per_wave == 16), "attention_prefill: split weights run with 16 rows a wave and no shared tiles (share=%d rows=%d)", share, rows_per_wave);
   ALOFA_REQUIRE(v_head < kv_heads && reinterpret_cast<uintptr_t>(out32) % 16 == 0, "attention_prefill: value head %d of %d; float rows 16-byte aligned", v_head, kv_heads);
   ALOFA_REQUIRE(n_tiles > 0 && heads > 0 && kv_heads > 0 && heads % kv_heads == 0,
                 "attention_prefill: tiles=%d heads=%d kv_heads=%d (kv_heads must divide heads)", n_tiles, heads, kv_heads);
@@ -530,6 +542,23 @@ extern "C" int alofa_attention_prefill_v(void* out, int64_t out_stride, const vo
   attention_prefill_kernel<DT, TEAMS, WPT, SHARE><<<GRID, 64 * WPT * TEAMS, 0, stream>>>(                                    \
       static_cast<bf16_t*>(out), out_stride, static_cast<const bf16_t*>(q), q_stride, static_cast<const bf16_t*>(k_cache), \
       static_cast<const bf16_t*>(v_cache), block_table, max_blocks, tiles, heads, kv_heads, bs_shift, window, scale, v_head, out32)
+#define ALOFA_PREFILL_SPLIT(DT)                                                                                               \
+  attention_prefill_kernel<DT, kTeams<DT>, 4, false, 16, 64, true><<<dim3(n_tiles, heads), 64 * 4 * kTeams<DT>, 0, stream>>>(  \
+      static_cast<bf16_t*>(out), out_stride, static_cast<const bf16_t*>(q), q_stride, static_cast<const bf16_t*>(k_cache), \
+      static_cast<const bf16_t*>(v_cache), block_table, max_blocks, tiles, heads, kv_heads, bs_shift, window, scale, v_head, out32)
+  if (split) {
+    switch (d / 16) {
+      case 1: ALOFA_PREFILL_SPLIT(1); break;
+      case 2: ALOFA_PREFILL_SPLIT(2); break;
+      case 3: ALOFA_PREFILL_SPLIT(3); break;
+      case 4: ALOFA_PREFILL_SPLIT(4); break;
+      case 6: ALOFA_PREFILL_SPLIT(6); break;
+      case 8: ALOFA_PREFILL_SPLIT(8); break;
+      case 16: ALOFA_PREFILL_SPLIT(16); break;
+    }
+    return check_launch("attention_prefill");
+  }
+#undef ALOFA_PREFILL_SPLIT
 #define ALOFA_PREFILL_AS32(DT, TEAMS, WPT, SHARE, GRID)                                                                       \
   attention_prefill_kernel<DT, TEAMS, WPT, SHARE, 32, (DT > 6 ? 32 : 64)><<<GRID, 64 * WPT * TEAMS, 0, stream>>>(            \
       static_cast<bf16_t*>(out), out_stride, static_cast<const bf16_t*>(q), q_stride, static_cast<const bf16_t*>(k_cache), \
@@ -575,5 +604,5 @@ extern "C" int alofa_attention_prefill(void* out, int64_t out_stride, const void
                                        int max_blocks, const int32_t* tiles, int n_tiles, int heads, int kv_heads, int d,
                                        int block_size, int window, float scale, int share, int rows_per_wave, hipStream_t stream) {
   return alofa_attention_prefill_v(out, out_stride, q, q_stride, k_cache, v_cache, block_table, max_blocks, tiles, n_tiles, heads, kv_heads, d, block_size, window,
-                                   scale, share, rows_per_wave, -1, nullptr, stream);
+                                   scale, share, rows_per_wave, -1, nullptr, 0, stream);
 }

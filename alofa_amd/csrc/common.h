@@ -29,6 +29,11 @@ __device__ __forceinline__ uint32_t pack_bf16x2(float a, float b) {
   return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_t));
 }
 
+// what pack_bf16x2 rounded away of a and b, as a second pair: the two pairs together keep sixteen bits of each
+__device__ __forceinline__ uint32_t pack_bf16x2_rest(float a, float b, uint32_t packed) {
+  return pack_bf16x2(a - __uint_as_float(packed << 16), b - __uint_as_float(packed & 0xffff0000u));
+}
+
 __device__ __forceinline__ bf16_t f32_to_bf16(float f) { return static_cast<bf16_t>(pack_bf16x2(f, 0.f) & 0xffffu); }
 
 template <typename T> __device__ __forceinline__ float load_f32(const T* p);

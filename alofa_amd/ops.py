@@ -655,7 +655,7 @@ def _attention_operands(out, q, k_cache, v_cache, block_table, heads, kv_heads, 
 def attention_decode(out, q, k_cache, v_cache, block_table, req_of_token, positions, heads, kv_heads, d, window, scale,
                      max_context: int, scratch: Optional[torch.Tensor], rows: Optional[torch.Tensor] = None,
                      rope: Optional[tuple] = None, n_splits: Optional[int] = None, hand_over: Optional[bool] = None,
-                     v_head: Optional[int] = None) -> None:
+                     v_head: Optional[int] = None, fine_weights: bool = False) -> None:
     """bfloat16 attention for tokens of requests that bring few tokens: every
     token of the batch, or the tokens ``rows`` (int32 indices into the batch).
     ``req_of_token`` None: every request brings one token and token i is request
@@ -668,7 +668,8 @@ def attention_decode(out, q, k_cache, v_cache, block_table, req_of_token, positi
     ``hand_over`` (default ``decode_hand_over``): the last of them to arrive combines their states,
     else the states go to ``scratch`` and a second kernel combines them.
     ``v_head``: every query head's weights meet the values of this one value head (the keys stay its own key head's).
-    ``out`` may be float32: the results are then stored unrounded."""
+    ``out`` may be float32: the results are then stored unrounded. ``fine_weights``: every softmax weight meets the values as two bfloat16
+    numbers, its rounding and what the rounding took away, so that sixteen bits of it count (twice the second product's instructions)."""
     T, bs = _attention_operands(out, q, k_cache, v_cache, block_table, heads, kv_heads, d)
     for n, t in (("req_of_token", req_of_token), ("positions", positions)):
         if t is None and n == "req_of_token":
@@ -712,7 +713,7 @@ def attention_decode(out, q, k_cache, v_cache, block_table, req_of_token, positi
     _call("alofa_attention_decode_v", _ptr(None if as32 else out), _L(_rows("out", out)), _ptr(scratch if floats else None), _ptr(q), _L(_rows("q", q)),
           _ptr(k_cache), _ptr(v_cache), _ptr(block_table), _I(block_table.shape[1]), _ptr(req_of_token), _ptr(positions), _ptr(rows),
           _I(n_tok), _I(heads), _I(kv_heads), _I(d), _I(bs), _I(int(window or 0)), _F(scale), _I(n_splits),
-          _ptr(cos), _ptr(sin), _ptr(slots), _I(int(hand_over)), _I(-1 if v_head is None else v_head), _ptr(out if as32 else None), _stream())
+          _ptr(cos), _ptr(sin), _ptr(slots), _I(int(hand_over)), _I(-1 if v_head is None else v_head), _ptr(out if as32 else None), _I(int(fine_weights)), _stream())
 
 
 def can_fuse_rope_into_decode(d: int) -> bool:
@@ -787,14 +788,15 @@ def pair_tiles(runs: list, window: Optional[int] = None, heads: Optional[int] = 
 
 
 def attention_prefill(out, q, k_cache, v_cache, block_table, tiles, heads, kv_heads, d, window, scale, share: int = 0,
-                      rows: int = 16, v_head: Optional[int] = None) -> None:
+                      rows: int = 16, v_head: Optional[int] = None, fine_weights: bool = False) -> None:
     """bfloat16 attention for portions of prompts. ``tiles`` is int32 [n, 2, 4]
     from ``pair_tiles``: per block up to two runs of rows, each (request index,
     first row, rows <= 64 or 0 for none, position of the first row). ``share``
     (from ``prefill_share``; the tiles were paired for its count of blocks):
     that many heads of a group are served from one staged tile. ``rows``: query rows a wave owns
     (from ``prefill_rows``; the tiles were paired for it too). ``v_head``: every query head's weights meet the values of this one
-    value head. ``out`` may be float32: the results are then stored unrounded."""
+    value head. ``out`` may be float32: the results are then stored unrounded. ``fine_weights`` (with ``share`` 0 and 16 ``rows``): every softmax
+    weight meets the values as two bfloat16 numbers, so that sixteen bits of it count."""
     T, bs = _attention_operands(out, q, k_cache, v_cache, block_table, heads, kv_heads, d)
     if d not in PREFILL_HEAD_DIMS:
         raise AlofaError("unsupported", "the prefill attention kernel is not built for this head size", f"head_dim={d} built={PREFILL_HEAD_DIMS}")
@@ -806,7 +808,7 @@ def attention_prefill(out, q, k_cache, v_cache, block_table, tiles, heads, kv_he
     as32 = out.dtype is torch.float32
     _call("alofa_attention_prefill_v", _ptr(None if as32 else out), _L(_rows("out", out)), _ptr(q), _L(_rows("q", q)), _ptr(k_cache), _ptr(v_cache),
           _ptr(block_table), _I(block_table.shape[1]), _ptr(tiles), _I(tiles.shape[0]), _I(heads), _I(kv_heads), _I(d), _I(bs),
-          _I(int(window or 0)), _F(scale), _I(share), _I(rows), _I(-1 if v_head is None else v_head), _ptr(out if as32 else None), _stream())
+          _I(int(window or 0)), _F(scale), _I(share), _I(rows), _I(-1 if v_head is None else v_head), _ptr(out if as32 else None), _I(int(fine_weights)), _stream())
 
 
 # ------------------------------------------------------------------ sampling

@@ -44,14 +44,15 @@ class RowPlan:
                 self.short_rows = torch.tensor([r for s in spans if s.n <= SHORT for r in range(s.row0, s.row0 + s.n)],
                                                dtype=torch.int32, device=self.device)
 
-    def tiles(self, heads: int, kv_heads: int, d: int, window):
+    def tiles(self, heads: int, kv_heads: int, d: int, window, plain: bool = False):
         """The runs as blocks of the prefill kernel for a mixer with these head counts, how many heads
         of a group share a block's tiles and how many rows a wave owns (all three depend on how many
-        blocks there are)."""
-        key = (heads, kv_heads, d, window)
+        blocks there are). ``plain``: every head has blocks of its own and a wave owns 16 rows (the
+        one form of the kernel that takes the weights in two parts)."""
+        key = (heads, kv_heads, d, window, plain)
         if key not in self._tiles:
-            share = ops.prefill_share(heads, kv_heads, d, len(self.long_runs))
-            rows = ops.prefill_rows(heads, kv_heads, d, share, len(self.long_runs))
+            share = 0 if plain else ops.prefill_share(heads, kv_heads, d, len(self.long_runs))
+            rows = 16 if plain else ops.prefill_rows(heads, kv_heads, d, share, len(self.long_runs))
             per_run = ops.prefill_blocks_per_run(heads, kv_heads, share, rows)
             self._tiles[key] = (torch.tensor(ops.pair_tiles(self.long_runs, window, per_run), dtype=torch.int32, device=self.device), share, rows)
         return self._tiles[key]

@@ -17,7 +17,8 @@ Mixing the weights is linear in what they are applied to: head h's result is sum
 unmixed weights applied to the values of value head c. In bfloat16, with pages of a power of two and heads of one size that the
 matrix-core attention kernels are built for, those kernels run once per value head (portions of prompts through the prefill kernel,
 single tokens through the decode kernel, as in ``paged_attend``) and leave A unrounded; one small kernel then mixes, turns back and
-gates. Every other case (float32, other sizes) runs the always-valid kernel, a block per row."""
+gates. The softmax weights are 32-bit numbers in this part: they meet the values as two bfloat16 numbers each, the rounding and what it
+took away (``fine_weights``), so that sixteen bits of every weight count. Every other case (float32, other sizes) runs the always-valid kernel, a block per row."""
 from __future__ import annotations
 
 import torch
@@ -114,11 +115,11 @@ class TalkingAttention(Mixer):
         one_each = ctx.max_q_len == 1 and plan.short_rows is None and plan.long_runs is None
         for c in range(self.kv_heads):
             if plan.long_runs is not None:
-                tiles, share, rows = plan.tiles(self.heads, self.kv_heads, self.d, self.window)
-                ops.attention_prefill(applied[c], q, kc, vc, table, tiles, *common, share=share, rows=rows, v_head=c)
+                tiles, share, rows = plan.tiles(self.heads, self.kv_heads, self.d, self.window, plain=True)
+                ops.attention_prefill(applied[c], q, kc, vc, table, tiles, *common, share=share, rows=rows, v_head=c, fine_weights=True)
             if plan.n_short:
                 ops.attention_decode(applied[c], q, kc, vc, table, None if one_each else ctx.req_of_token, ctx.positions, *common,
-                                     ctx.max_context, partial, rows=plan.short_rows, v_head=c)
+                                     ctx.max_context, partial, rows=plan.short_rows, v_head=c, fine_weights=True)
         ops.talk_mix(attn, applied, ctx.positions, self.heads, self.kv_heads, self.dv, self.talk, v_table, gate)
 
     def forward(self, ctx, where, x, residual, out=None):

@@ -123,6 +123,7 @@ def retotar_dirs(tmp_path_factory):
     out = {}
     for name, cfg in RETOTAR.items():
         d = tmp_path_factory.mktemp(f"retotar_{name}")
-        write_random_model(cfg, d, seed=4000 + ord(name))
+        # (F: of a few seeds the one with which the routers' calls stay clear at most positions, so that most positions are compared in bfloat16)
+        write_random_model(cfg, d, seed=11 if name == "F" else 4000 + ord(name))
         out[name] = d
     return out

@@ -74,6 +74,14 @@ RETOTAR = {
         (_lightning(3, 9, 7, (0.85, 0.9, 0.95)), _moe(3, 2, 14, identity=1, groups=(2, 1))),
         (_mlstm(5, 5, 3, 8.0), _moe(7, 2, 22, identity=2, groups=(3, 2))),
         (_attention(10, 5, 10, 6, 10, 777.0, 0.35, mask=12, kv_from=0), None)]),
+    # query/key and value heads of one size in steps of sixteen, which the matrix-core attention kernels take in bfloat16: six heads over
+    # three with a short window, four over one without a window, and a layer that reads the first one's pages through a longer window
+    "F": _config(173, 96, 1e-5, 0.8, [
+        (_attention(6, 3, 32, 32, 8, 10000.0, 0.2, mask=20, factor=4.0), _moe(6, 2, 32, identity=2, groups=(2, 1))),
+        (_lightning(3, 16, 32, (0.8, 0.9, 0.97)), None),
+        (_attention(4, 1, 16, 16, 16, 5000.0, 0.3), _moe(4, 1, 16)),
+        (_attention(6, 3, 32, 32, 8, 10000.0, 0.25, mask=33, factor=4.0, kv_from=0), _moe(6, 2, 32, identity=2, groups=(2, 1))),
+        (_mlstm(2, 16, 16, 9.0), None)]),
 }
 
 

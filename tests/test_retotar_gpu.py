@@ -15,7 +15,7 @@ from retotar_cases import RETOTAR, clear_calls, clear_ids, plain_logits, plain_m
 pytestmark = pytest.mark.gpu
 
 DTYPES = ["float32", "bfloat16"]
-LENGTHS = {"A": 100, "B": 75, "C": 120, "D": 150, "E": 90}
+LENGTHS = {"A": 100, "B": 75, "C": 120, "D": 150, "E": 90, "F": 140}
 
 
 @pytest.fixture(scope="module")
@@ -93,7 +93,7 @@ def _one_layer(cfg, i):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("name,layer", [("A", 0), ("A", 1), ("A", 2), ("B", 1), ("C", 2), ("D", 1), ("D", 3), ("E", 2), ("E", 3)])
+@pytest.mark.parametrize("name,layer", [("A", 0), ("A", 1), ("A", 2), ("B", 1), ("C", 2), ("D", 1), ("D", 3), ("E", 2), ("E", 3), ("F", 0), ("F", 2)])
 def test_every_mixer_alone(tmp_path, name, layer, dtype):
     """One layer, with and without its feed-forward: whole, then token by token, then in portions."""
     from alofa_amd.replay import Replayer
@@ -183,7 +183,8 @@ def _variant(cfg, out_dir, seed, change):
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("window", [15, 16, 17, 31, 33, 1, 2])
-def test_windows_around_page_borders_with_keys_that_decide(tmp_path, window, dtype):
+@pytest.mark.parametrize("base", ["A", "F"])      # (F: head sizes that run on the matrix cores in bfloat16)
+def test_windows_around_page_borders_with_keys_that_decide(tmp_path, base, window, dtype):
     """Scores scaled up until single keys carry nearly all the weight, and windows that end on a page's border, one before and one
     behind (pages of 16), and of one and two keys: a key too many or too few at a window's edge shows in every logit, in
     prompts' portions and in decoding. One layer reads the other's pages through a window twice as long."""
@@ -192,8 +193,8 @@ def test_windows_around_page_borders_with_keys_that_decide(tmp_path, window, dty
     def change(cfg):
         first, last = cfg["layers"][0]["mixer"], cfg["layers"][3]["mixer"]
         first["mask"]["size"], last["mask"]["size"] = window, 2 * window
-        first["scale"], last["scale"] = 2.5, 3.0
-    d = _variant(RETOTAR["A"], tmp_path / "w", 500 + window, change)
+        first["scale"], last["scale"] = 40.0 / first["dim"], 48.0 / last["dim"]      # (unit-norm heads: the largest possible score is scale x dim)
+    d = _variant(RETOTAR[base], tmp_path / "w", 500 + window, change)
     cfg, w = plain_model(str(d))
     ids = clear_ids(str(d), 130)
     # (the weights do concentrate: the largest softmax weight of the last query, somewhere among the first layer's heads, is large)
@@ -212,14 +213,15 @@ def test_windows_around_page_borders_with_keys_that_decide(tmp_path, window, dty
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-def test_a_far_key_that_decides(tmp_path, dtype):
+@pytest.mark.parametrize("base,attention,other", [("C", 2, 0), ("F", 2, 1)])
+def test_a_far_key_that_decides(tmp_path, base, attention, other, dtype):
     """No window (every key is kept), scores scaled up: single keys hundreds of tokens back and across many pages decide."""
     from alofa_amd.replay import Replayer
 
     def change(cfg):
-        cfg["layers"] = [cfg["layers"][2], cfg["layers"][0]]      # attention without a window, then the linear attention
+        cfg["layers"] = [cfg["layers"][attention], cfg["layers"][other]]      # attention without a window, then the linear attention
         cfg["layers"][0]["mixer"]["scale"] = 2.0
-    d = _variant(RETOTAR["C"], tmp_path / "far", 600, change)
+    d = _variant(RETOTAR[base], tmp_path / "far", 600, change)
     ids = clear_ids(str(d), 330)
     r = Replayer(d, dtype, 384, max_requests=2)
     compare(collect(r, portions("p", ids, sizes=(150, 2, 61, 17, 3)))["p"], d, ids, dtype, "far key, portions")
@@ -246,6 +248,27 @@ def test_an_old_token_in_the_memories(tmp_path, dtype):
     compare(collect(r, portions("p", ids, sizes=(130, 2, 61, 17, 3)))["p"], d, ids, dtype, "old token, portions")
     collect(r, whole("other", random_ids(5, 50, RETOTAR["A"]["vocab"])))
     compare(collect(r, bulk_and_tail("t", ids, tail=60))["t"], d, ids, dtype, "old token, decoding")
+
+
+def test_heads_of_one_size_run_on_the_matrix_cores(replayers, retotar_dirs, monkeypatch):
+    """In bfloat16 the attention layers of F go through the matrix-core kernels, once per value head, and the kernel that mixes afterwards;
+    in float32, and with heads of two sizes, through the kernel that takes a block per row."""
+    from alofa_amd import ops
+    calls = {"talk_mix": 0, "talking_attention": 0}
+
+    def counted(name):
+        real = getattr(ops, name)
+
+        def call(*a, **k):
+            calls[name] += 1
+            return real(*a, **k)
+        return call
+    for name in calls:
+        monkeypatch.setattr(ops, name, counted(name))
+    for model, dtype, mixed, per_row in (("F", "bfloat16", 3, 0), ("F", "float32", 0, 3), ("A", "bfloat16", 0, 2)):
+        calls.update(talk_mix=0, talking_attention=0)
+        collect(replayers(model, dtype), whole("m", random_ids(3, 70, RETOTAR[model]["vocab"])))
+        assert (calls["talk_mix"], calls["talking_attention"]) == (mixed, per_row), (model, dtype, calls)
 
 
 def test_greedy_generation_through_the_engine(retotar_dirs):

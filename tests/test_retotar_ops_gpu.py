@@ -89,11 +89,11 @@ def test_attention_over_shuffled_pages_in_portions(H, G, d, dv, dims, window, dt
             for c in range(G):
                 if runs:
                     tiles = torch.tensor(ops.pair_tiles(runs, window, H), dtype=torch.int32, device=DEV)
-                    ops.attention_prefill(applied[c], rows[:, :H * d], kc, vc, table.to(DEV), tiles, H, G, d, window, scale, v_head=c)
+                    ops.attention_prefill(applied[c], rows[:, :H * d], kc, vc, table.to(DEV), tiles, H, G, d, window, scale, v_head=c, fine_weights=True)
                 if short:
                     floats = ops.decode_scratch_floats(len(short), H, G, d, 128, window)
                     ops.attention_decode(applied[c], rows[:, :H * d], kc, vc, table.to(DEV), req, positions, H, G, d, window, scale, 128,
-                                         torch.empty(max(floats, 1), device=DEV), rows=torch.tensor(short, dtype=torch.int32, device=DEV), v_head=c)
+                                         torch.empty(max(floats, 1), device=DEV), rows=torch.tensor(short, dtype=torch.int32, device=DEV), v_head=c, fine_weights=True)
             out_fast = torch.empty_like(out)
             ops.talk_mix(out_fast, applied, positions, H, G, dv, dev(talk.numpy()), v_t, rows[:, width:])
         at = 0
