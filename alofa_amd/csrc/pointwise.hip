@@ -63,6 +63,46 @@ __global__ void __launch_bounds__(256) layernorm_add_kernel(float* __restrict__ 
   }
 }
 
+// The same, and then the layer norm (w2, b2) of the row as it now stands, left in `out`: the norm behind one sub-layer and the one in front
+// of the next in one launch. Every thread reads back what it wrote itself; the sums are those of the two kernels run one after the other.
+template <typename TO, typename Acc>
+__global__ void __launch_bounds__(256) layernorm_add_norm_kernel(float* __restrict__ residual, const float* __restrict__ x, const float* __restrict__ w,
+                                                                 const float* __restrict__ b, float eps, TO* __restrict__ out, const float* __restrict__ w2,
+                                                                 const float* __restrict__ b2, float eps2, int width) {
+  __shared__ Acc scratch[4];
+  const int r = blockIdx.x;
+  const float* src = x + static_cast<int64_t>(r) * width;
+  float* dst = residual + static_cast<int64_t>(r) * width;
+  Acc s = 0;
+  for (int c = threadIdx.x; c < width; c += 256) s += static_cast<Acc>(src[c]);
+  const Acc mean = block_sum<Acc, 256>(s, scratch) / static_cast<Acc>(width);
+  Acc ss = 0;
+  for (int c = threadIdx.x; c < width; c += 256) {
+    const Acc d = static_cast<Acc>(src[c]) - mean;
+    ss += d * d;
+  }
+  const Acc var = block_sum<Acc, 256>(ss, scratch) / static_cast<Acc>(width);
+  const Acc inv = static_cast<Acc>(1) / sqrt(var + static_cast<Acc>(eps));
+  Acc s2 = 0;
+  for (int c = threadIdx.x; c < width; c += 256) {
+    const Acc y = (static_cast<Acc>(src[c]) - mean) * inv * static_cast<Acc>(w[c]) + static_cast<Acc>(b[c]);
+    const float now = static_cast<float>(static_cast<Acc>(dst[c]) + y);
+    dst[c] = now;
+    s2 += static_cast<Acc>(now);
+  }
+  const Acc mean2 = block_sum<Acc, 256>(s2, scratch) / static_cast<Acc>(width);
+  Acc ss2 = 0;
+  for (int c = threadIdx.x; c < width; c += 256) {
+    const Acc d = static_cast<Acc>(dst[c]) - mean2;
+    ss2 += d * d;
+  }
+  const Acc var2 = block_sum<Acc, 256>(ss2, scratch) / static_cast<Acc>(width);
+  const Acc inv2 = static_cast<Acc>(1) / sqrt(var2 + static_cast<Acc>(eps2));
+  TO* normed = out + static_cast<int64_t>(r) * width;
+  for (int c = threadIdx.x; c < width; c += 256)
+    store_f32(normed + c, static_cast<float>((static_cast<Acc>(dst[c]) - mean2) * inv2 * static_cast<Acc>(w2[c]) + static_cast<Acc>(b2[c])));
+}
+
 // out[t, c] += w[t] * x[t, c]: a row handed on with a weight of its own (float rows out, rows of any type in).
 template <typename T, typename Acc>
 __global__ void __launch_bounds__(256) add_row_scaled_kernel(float* __restrict__ out, const T* __restrict__ x, int64_t x_stride, const float* __restrict__ w,
@@ -274,6 +314,17 @@ extern "C" int alofa_layernorm_add(float* residual, const float* x, const float*
   if (exact) layernorm_add_kernel<double><<<n_rows, 256, 0, stream>>>(residual, x, w, b, width, eps);
   else layernorm_add_kernel<float><<<n_rows, 256, 0, stream>>>(residual, x, w, b, width, eps);
   return check_launch("layernorm_add");
+}
+
+extern "C" int alofa_layernorm_add_norm(float* residual, const float* x, const float* w, const float* b, float eps, void* out, int out_dtype, const float* w2,
+                                        const float* b2, float eps2, int n_rows, int width, int exact, hipStream_t stream) {
+  ALOFA_REQUIRE(n_rows >= 0 && width > 0 && eps > 0.f && eps2 > 0.f, "layernorm_add_norm: bad sizes (rows=%d width=%d)", n_rows, width);
+  ALOFA_REQUIRE(!exact || out_dtype == kF32, "layernorm_add_norm: the exact path is float32");
+  if (n_rows == 0) return 0;
+  if (exact) layernorm_add_norm_kernel<float, double><<<n_rows, 256, 0, stream>>>(residual, x, w, b, eps, static_cast<float*>(out), w2, b2, eps2, width);
+  else if (out_dtype == kF32) layernorm_add_norm_kernel<float, float><<<n_rows, 256, 0, stream>>>(residual, x, w, b, eps, static_cast<float*>(out), w2, b2, eps2, width);
+  else layernorm_add_norm_kernel<bf16_t, float><<<n_rows, 256, 0, stream>>>(residual, x, w, b, eps, static_cast<bf16_t*>(out), w2, b2, eps2, width);
+  return check_launch("layernorm_add_norm");
 }
 
 extern "C" int alofa_add_row_scaled(float* out, const void* x, int64_t x_stride, int dtype, const float* w, int64_t rows, int width, int exact, hipStream_t stream) {

@@ -1030,6 +1030,24 @@ def layernorm_add(residual: torch.Tensor, x: torch.Tensor, w: torch.Tensor, b: t
     _call("alofa_layernorm_add", _ptr(residual), _ptr(x), _ptr(w), _ptr(b), _I(n), _I(h), _F(eps), _I(int(exact)), _stream())
 
 
+def layernorm_add_norm(residual: torch.Tensor, x: torch.Tensor, w: torch.Tensor, b: torch.Tensor, eps: float, out: torch.Tensor, w2: torch.Tensor,
+                       b2: torch.Tensor, eps2: float, exact: bool = False) -> None:
+    """``layernorm_add`` and then ``out[r]`` = the layer norm (w2, b2, eps2) of the row as it now stands, in one launch: the norm behind one
+    sub-layer and the one in front of the next. ``out`` [n, h] contiguous in the activation dtype."""
+    for n_, t in (("residual", residual), ("x", x)):
+        _gpu(n_, t, torch.float32, 2), _contig(n_, t)
+    for n_, t in (("w", w), ("b", b), ("w2", w2), ("b2", b2)):
+        _gpu(n_, t, torch.float32, 1), _contig(n_, t)
+    _gpu("out", out, None, 2), _contig("out", out)
+    n, h = residual.shape
+    if tuple(x.shape) != (n, h) or tuple(out.shape) != (n, h) or any(t.shape[0] != h for t in (w, b, w2, b2)):
+        raise AlofaError("shape_mismatch", "norm width does not fit", f"residual={tuple(residual.shape)} x={tuple(x.shape)} out={tuple(out.shape)} w={tuple(w.shape)}")
+    if exact and out.dtype is not torch.float32:
+        raise AlofaError("invalid_argument", "the exact path is float32")
+    _call("alofa_layernorm_add_norm", _ptr(residual), _ptr(x), _ptr(w), _ptr(b), _F(eps), _ptr(out), _I(dtype_code(out)), _ptr(w2), _ptr(b2), _F(eps2),
+          _I(n), _I(h), _I(int(exact)), _stream())
+
+
 def add_row_scaled(out: torch.Tensor, x: torch.Tensor, w: torch.Tensor, exact: bool = False) -> None:
     """out[t] += w[t] * x[t]: ``out`` float32 [T, h] contiguous, ``x`` [T, h] rows of any type (row strides allowed), ``w`` float32 [T]."""
     _gpu("out", out, torch.float32, 2), _gpu("x", x, None, 2), _gpu("w", w, torch.float32, 1), _contig("out", out), _contig("w", w)

@@ -239,7 +239,8 @@ class SandwichBlock(Block):
     """a += post0(mixer(pre0(a))), then, where the layer has a feed-forward, a += post1(feed_forward(pre1(a))).
     It reads the layer's parts ``mixer``, ``feed_forward`` (may be None) and ``norms``: (pre0, post0) or (pre0, post0, pre1, post1).
     Mixer and feed-forward leave their results apart (``out=``); a layer norm behind a sub-layer is applied by the launch that adds
-    to the stream, any other norm runs where the result lies and a sum follows."""
+    to the stream, any other norm runs where the result lies and a sum follows. Where the norm behind the mixer and the one in front of
+    the feed-forward are both layer norms, one launch adds and leaves the feed-forward's input."""
 
     @classmethod
     def layer_tensors(cls, layer) -> dict:
@@ -278,9 +279,15 @@ class SandwichBlock(Block):
         apart = ctx.scratch("sub_out", tuple(hidden.shape), torch.float32)
         self.norms[0].forward(buf, hidden)
         self.mixer.forward(ctx, (entry, 0), buf, hidden, out=apart)
-        self._join(hidden, apart, self.norms[1])
-        if self.feed_forward is not None:
-            self.norms[2].forward(buf, hidden)
+        if self.feed_forward is None:
+            self._join(hidden, apart, self.norms[1])
+        else:
+            behind, front = self.norms[1].as_layernorm(), self.norms[2].as_layernorm()
+            if behind is not None and front is not None and FUSE_SUMS:
+                ops.layernorm_add_norm(hidden, apart, *behind, buf, *front, exact=self.rt.exact)
+            else:
+                self._join(hidden, apart, self.norms[1])
+                self.norms[2].forward(buf, hidden)
             self.feed_forward.forward(ctx, buf, hidden, out=apart)
             self._join(hidden, apart, self.norms[3])
 

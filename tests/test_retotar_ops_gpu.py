@@ -187,6 +187,17 @@ def test_the_norm_that_adds_and_the_row_handed_on():
             out = dev(res)
             ops.layernorm_add(out, dev(x), dev(w), dev(b), 1e-5, exact)
             assert (out.cpu().double() - want).abs().max() <= (2e-6 if exact else 2e-5)
+        # the norm in front of the next sub-layer in the same launch: the stream as after the sum, and its norm
+        w2, b2 = rng.normal(1, 0.2, width), rng.normal(0, 0.5, width)
+        for dtype in (torch.float32, torch.bfloat16):
+            out, normed = dev(res), torch.empty(9, width, dtype=dtype, device=DEV)
+            ops.layernorm_add_norm(out, dev(x), dev(w), dev(b), 1e-5, normed, dev(w2), dev(b2), 1e-6, exact=dtype is torch.float32)
+            assert (out.cpu().double() - want).abs().max() <= 2e-5
+            after = pt.layer_norm(out.cpu().double(), f32(w2), f32(b2), 1e-6)
+            assert (normed.cpu().double() - after).abs().max() <= (1e-5 if dtype is torch.float32 else 3e-2)
+            apart = torch.empty(9, width, dtype=dtype, device=DEV)
+            ops.layernorm(apart, out, dev(w2), dev(b2), 1e-6, dtype is torch.float32)
+            assert torch.equal(apart, normed)      # (the same sums as the two launches one after the other)
         scale = rng.normal(0, 1, 9)
         scale[3] = 0.0
         for dtype in (torch.float32, torch.bfloat16):
