@@ -93,7 +93,7 @@ __global__ void __launch_bounds__(64 * NW) attention_decode_kernel(
     int64_t q_stride, bf16_t* __restrict__ k_cache, bf16_t* __restrict__ v_cache,
     const int32_t* __restrict__ block_table, int max_blocks, const int32_t* __restrict__ req_of_token,
     const int32_t* __restrict__ positions, const int32_t* __restrict__ rows, int heads, int kv_heads,
-    int bs_shift, int window, float scale, RopeArgs rope, int* __restrict__ counters, int v_head, float* __restrict__ out32) {
+    int bs_shift, int window, float scale, RopeArgs rope, int* __restrict__ counters, int v_head, float* __restrict__ out32, int value_heads, int64_t plane) {
   static_assert(!kRope || DT % 4 == 0, "the rotation needs a channel and its partner in the same lane: d a multiple of 64");
   constexpr int d = DT * 16;
   constexpr int DS = (d + 31) / 32;            // steps of 32 along d in the first product
@@ -103,7 +103,13 @@ __global__ void __launch_bounds__(64 * NW) attention_decode_kernel(
   const int group = heads / kv_heads;
   const int chunks = (group + kHeadsPerBlock - 1) / kHeadsPerBlock;
   // the tokens served are rows[0..gridDim.x) of the packed batch, or all of it
-  const int t = rows ? rows[blockIdx.x] : blockIdx.x;
+  // (value_heads > 0: blockIdx.x counts (token, value head) pairs: every value head in turn serves all key heads, and its results go to a plane of their own)
+  const int served = value_heads > 0 ? blockIdx.x / value_heads : blockIdx.x;
+  if (value_heads > 0) {
+    v_head = blockIdx.x % value_heads;
+    out32 += static_cast<int64_t>(v_head) * plane;
+  }
+  const int t = rows ? rows[served] : served;
   const int hk = blockIdx.y / chunks, h0 = (blockIdx.y % chunks) * kHeadsPerBlock;
   const int hv = v_head >= 0 ? v_head : hk;      // the value head whose values the weights meet (v_head >= 0: one for all key heads)
   const int wave = threadIdx.x / 64, lane = threadIdx.x % 64;
@@ -481,9 +487,11 @@ __global__ void __launch_bounds__(64 * NW) attention_decode_kernel(
 __global__ void __launch_bounds__(256) attention_merge_kernel(bf16_t* __restrict__ out, int64_t out_stride,
                                                               const float* __restrict__ partial,
                                                               const int32_t* __restrict__ rows, int heads, int d,
-                                                              int n_splits, float* __restrict__ out32) {
+                                                              int n_splits, float* __restrict__ out32, int value_heads, int64_t plane) {
   __shared__ float sums[4][256];
-  const int t = rows ? rows[blockIdx.x] : blockIdx.x, h = blockIdx.y, lane = threadIdx.x % 64;
+  const int served = value_heads > 0 ? blockIdx.x / value_heads : blockIdx.x;
+  if (value_heads > 0) out32 += static_cast<int64_t>(blockIdx.x % value_heads) * plane;
+  const int t = rows ? rows[served] : served, h = blockIdx.y, lane = threadIdx.x % 64;
   const int wave = threadIdx.x / 64, waves = blockDim.x / 64;
   const float* src = partial + (static_cast<int64_t>(blockIdx.x) * heads + h) * n_splits * (d + 2);
   // lane s holds part s's maximum and sum (n_splits <= 64)
@@ -554,8 +562,12 @@ extern "C" int alofa_attention_decode_v(void* out, int64_t out_stride, float* pa
                                         int max_blocks, const int32_t* req_of_token, const int32_t* positions,
                                         const int32_t* rows, int tokens, int heads, int kv_heads, int d, int block_size, int window,
                                         float scale, int n_splits, const float* cos_t, const float* sin_t, const int64_t* slots,
-                                        int hand_over, int v_head, float* out32, int split, hipStream_t stream) {
+                                        int hand_over, int v_head, float* out32, int split, int value_heads, int64_t plane, hipStream_t stream) {
   ALOFA_REQUIRE(!split || !cos_t, "attention_decode: split weights and the rotary variant do not go together");
+  // value_heads > 0: all of them in one launch, value head c's results in out32 + c * plane; `tokens` then counts (token, value head) pairs
+  // wherever it sizes scratch, workspace and grid
+  ALOFA_REQUIRE(value_heads == 0 || (value_heads == kv_heads && out32 && v_head < 0 && !cos_t && plane > 0), "attention_decode: all %d value heads in one launch need float rows and no value head named", kv_heads);
+  if (value_heads > 0) tokens *= value_heads;
   ALOFA_REQUIRE(v_head < kv_heads && (v_head < 0 || !cos_t), "attention_decode: value head %d of %d (and none with the rotary variant)", v_head, kv_heads);
   ALOFA_REQUIRE(tokens > 0 && heads > 0 && kv_heads > 0 && heads % kv_heads == 0,
                 "attention_decode: tokens=%d heads=%d kv_heads=%d (kv_heads must divide heads)", tokens, heads, kv_heads);
@@ -585,11 +597,11 @@ extern "C" int alofa_attention_decode_v(void* out, int64_t out_stride, float* pa
   if (split && !ROPE) attention_decode_kernel<DT, NW, false, true><<<grid, 64 * NW, 0, stream>>>(                         \
       static_cast<bf16_t*>(out), out_stride, partial, static_cast<const bf16_t*>(q), q_stride,                            \
       static_cast<bf16_t*>(k_cache), static_cast<bf16_t*>(v_cache), block_table, max_blocks, req_of_token,                \
-      positions, rows, heads, kv_heads, bs_shift, window, scale, rope, counters, v_head, out32);                          \
+      positions, rows, heads, kv_heads, bs_shift, window, scale, rope, counters, v_head, out32, value_heads, plane);       \
   else attention_decode_kernel<DT, NW, ROPE><<<grid, 64 * NW, 0, stream>>>(                                                    \
       static_cast<bf16_t*>(out), out_stride, partial, static_cast<const bf16_t*>(q), q_stride,                            \
       static_cast<bf16_t*>(k_cache), static_cast<bf16_t*>(v_cache), block_table, max_blocks, req_of_token,                \
-      positions, rows, heads, kv_heads, bs_shift, window, scale, rope, counters, v_head, out32)
+      positions, rows, heads, kv_heads, bs_shift, window, scale, rope, counters, v_head, out32, value_heads, plane)
   if (fused) {
     switch (d / 64) {
       case 1: ALOFA_DECODE(4, 8, true); break;
@@ -621,7 +633,7 @@ extern "C" int alofa_attention_decode_v(void* out, int64_t out_stride, float* pa
   if (check_launch("attention_decode")) return 1;
   if (n_splits > 1 && !counters) {
     // (one wave up to sixteen parts, whose loads are all on their way at once; four beyond)
-    attention_merge_kernel<<<dim3(tokens, heads), n_splits <= 16 ? 64 : 256, 0, stream>>>(static_cast<bf16_t*>(out), out_stride, partial, rows, heads, d, n_splits, out32);
+    attention_merge_kernel<<<dim3(tokens, heads), n_splits <= 16 ? 64 : 256, 0, stream>>>(static_cast<bf16_t*>(out), out_stride, partial, rows, heads, d, n_splits, out32, value_heads, plane);
     return check_launch("attention_merge");
   }
   return 0;
@@ -634,5 +646,5 @@ extern "C" int alofa_attention_decode(void* out, int64_t out_stride, float* part
                                       float scale, int n_splits, const float* cos_t, const float* sin_t, const int64_t* slots,
                                       int hand_over, hipStream_t stream) {
   return alofa_attention_decode_v(out, out_stride, partial, q, q_stride, k_cache, v_cache, block_table, max_blocks, req_of_token, positions, rows, tokens,
-                                  heads, kv_heads, d, block_size, window, scale, n_splits, cos_t, sin_t, slots, hand_over, -1, nullptr, 0, stream);
+                                  heads, kv_heads, d, block_size, window, scale, n_splits, cos_t, sin_t, slots, hand_over, -1, nullptr, 0, 0, 0, stream);
 }

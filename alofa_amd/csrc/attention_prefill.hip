@@ -67,7 +67,7 @@ __global__ void __launch_bounds__(64 * WPT * TEAMS, (RW == 32 && 64 * WPT * TEAM
     bf16_t* __restrict__ out, int64_t out_stride, const bf16_t* __restrict__ q, int64_t q_stride,
     const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache, const int32_t* __restrict__ block_table,
     int max_blocks, const int32_t* __restrict__ tiles, int heads, int kv_heads, int bs_shift, int window,
-    float scale, int v_head, float* __restrict__ out32) {
+    float scale, int v_head, float* __restrict__ out32, int value_heads, int64_t plane) {
   constexpr int d = DT * 16;
   constexpr int BKV = KT;
   static_assert(KT == 64 || (KT == 32 && RW == 32), "tiles of 64 keys, or of 32 with 32 rows a wave");
@@ -99,9 +99,15 @@ __global__ void __launch_bounds__(64 * WPT * TEAMS, (RW == 32 && 64 * WPT * TEAM
   const int hk = kShare ? blockIdx.y / chunks : blockIdx.y / group;
   const bool head_ok = !kShare || (blockIdx.y % chunks) * WPT + wave < group;
   const int head = kShare ? hk * group + (head_ok ? (blockIdx.y % chunks) * WPT + wave : 0) : blockIdx.y;
+  // (value_heads > 0: blockIdx.x counts (pair of runs, value head): every value head in turn serves all key heads, and its results go to a plane of their own)
+  const int pair = value_heads > 0 ? blockIdx.x / value_heads : blockIdx.x;
+  if (value_heads > 0) {
+    v_head = blockIdx.x % value_heads;
+    out32 += static_cast<int64_t>(v_head) * plane;
+  }
   const int hv = v_head >= 0 ? v_head : hk;      // the value head whose values the weights meet (v_head >= 0: one for all key heads)
   for (int part = 0; part < 2; ++part) {
-  const int32_t* tile = tiles + 8 * blockIdx.x + 4 * part;
+  const int32_t* tile = tiles + 8 * pair + 4 * part;
   // kShare: the block takes rows RW z .. of the run (fewer at the run's end; none: the block has nothing to do in this run)
   const int sub = kShare ? RW * blockIdx.z : 0;
   const int req = tile[0], row0 = tile[1] + sub, pos0 = tile[3] + sub;
@@ -518,7 +524,10 @@ extern "C" int alofa_attention_prefill_v(void* out, int64_t out_stride, const vo
                                          const void* k_cache, const void* v_cache, const int32_t* block_table,
                                          int max_blocks, const int32_t* tiles, int n_tiles, int heads, int kv_heads, int d,
                                          int block_size, int window, float scale, int share, int rows_per_wave, int v_head, float* out32, int split,
-                                         hipStream_t stream) {
+                                         int value_heads, int64_t plane, hipStream_t stream) {
+  // value_heads > 0: all of them in one launch, value head c's results in out32 + c * plane
+  ALOFA_REQUIRE(value_heads == 0 || (value_heads == kv_heads && out32 && v_head < 0 && plane > 0 && plane % 4 == 0), "attention_prefill: all %d value heads in one launch need float rows and no value head named", kv_heads);
+  if (value_heads > 0) n_tiles *= value_heads;      // (the grid's first dimension)
   ALOFA_REQUIRE(!split || (share == 0 && rows_per_wave == 16), "attention_prefill: split weights run with 16 rows a wave and no shared tiles (share=%d rows=%d)", share, rows_per_wave);
   ALOFA_REQUIRE(v_head < kv_heads && reinterpret_cast<uintptr_t>(out32) % 16 == 0, "attention_prefill: value head %d of %d; float rows 16-byte aligned", v_head, kv_heads);
   ALOFA_REQUIRE(n_tiles > 0 && heads > 0 && kv_heads > 0 && heads % kv_heads == 0,
@@ -541,11 +550,11 @@ extern "C" int alofa_attention_prefill_v(void* out, int64_t out_stride, const vo
 #define ALOFA_PREFILL_AS(DT, TEAMS, WPT, SHARE, GRID)                                                                         \
   attention_prefill_kernel<DT, TEAMS, WPT, SHARE><<<GRID, 64 * WPT * TEAMS, 0, stream>>>(                                    \
       static_cast<bf16_t*>(out), out_stride, static_cast<const bf16_t*>(q), q_stride, static_cast<const bf16_t*>(k_cache), \
-      static_cast<const bf16_t*>(v_cache), block_table, max_blocks, tiles, heads, kv_heads, bs_shift, window, scale, v_head, out32)
+      static_cast<const bf16_t*>(v_cache), block_table, max_blocks, tiles, heads, kv_heads, bs_shift, window, scale, v_head, out32, value_heads, plane)
 #define ALOFA_PREFILL_SPLIT(DT)                                                                                               \
   attention_prefill_kernel<DT, kTeams<DT>, 4, false, 16, 64, true><<<dim3(n_tiles, heads), 64 * 4 * kTeams<DT>, 0, stream>>>(  \
       static_cast<bf16_t*>(out), out_stride, static_cast<const bf16_t*>(q), q_stride, static_cast<const bf16_t*>(k_cache), \
-      static_cast<const bf16_t*>(v_cache), block_table, max_blocks, tiles, heads, kv_heads, bs_shift, window, scale, v_head, out32)
+      static_cast<const bf16_t*>(v_cache), block_table, max_blocks, tiles, heads, kv_heads, bs_shift, window, scale, v_head, out32, value_heads, plane)
   if (split) {
     switch (d / 16) {
       case 1: ALOFA_PREFILL_SPLIT(1); break;
@@ -562,7 +571,7 @@ extern "C" int alofa_attention_prefill_v(void* out, int64_t out_stride, const vo
 #define ALOFA_PREFILL_AS32(DT, TEAMS, WPT, SHARE, GRID)                                                                       \
   attention_prefill_kernel<DT, TEAMS, WPT, SHARE, 32, (DT > 6 ? 32 : 64)><<<GRID, 64 * WPT * TEAMS, 0, stream>>>(            \
       static_cast<bf16_t*>(out), out_stride, static_cast<const bf16_t*>(q), q_stride, static_cast<const bf16_t*>(k_cache), \
-      static_cast<const bf16_t*>(v_cache), block_table, max_blocks, tiles, heads, kv_heads, bs_shift, window, scale, v_head, out32)
+      static_cast<const bf16_t*>(v_cache), block_table, max_blocks, tiles, heads, kv_heads, bs_shift, window, scale, v_head, out32, value_heads, plane)
 #define ALOFA_PREFILL_WIDE32(DT, WPT)                                                                            \
   if (width == WPT) ALOFA_PREFILL_AS32(DT, (kShareTeams<DT>), WPT, true, dim3(n_tiles, kv_heads * chunks, 2))
 #define ALOFA_PREFILL32(DT)                                                                         \
@@ -604,5 +613,5 @@ extern "C" int alofa_attention_prefill(void* out, int64_t out_stride, const void
                                        int max_blocks, const int32_t* tiles, int n_tiles, int heads, int kv_heads, int d,
                                        int block_size, int window, float scale, int share, int rows_per_wave, hipStream_t stream) {
   return alofa_attention_prefill_v(out, out_stride, q, q_stride, k_cache, v_cache, block_table, max_blocks, tiles, n_tiles, heads, kv_heads, d, block_size, window,
-                                   scale, share, rows_per_wave, -1, nullptr, 0, stream);
+                                   scale, share, rows_per_wave, -1, nullptr, 0, 0, 0, stream);
 }

@@ -652,10 +652,20 @@ def _attention_operands(out, q, k_cache, v_cache, block_table, heads, kv_heads, 
     return T, bs
 
 
+def _value_planes(out, all_value_heads: bool, v_head, kv_heads: int) -> int:
+    """How many planes ``out`` has, one per value head (0: rows of one attention result)."""
+    if not all_value_heads:
+        return 0
+    if v_head is not None or out.dtype is not torch.float32 or out.dim() != 3 or out.shape[0] != kv_heads or not out.is_contiguous():
+        raise AlofaError("invalid_argument", "all value heads in one launch: float32 [kv_heads, T, heads * d], and no value head named",
+                         f"out={tuple(out.shape)} dtype={out.dtype} v_head={v_head} kv_heads={kv_heads}")
+    return kv_heads
+
+
 def attention_decode(out, q, k_cache, v_cache, block_table, req_of_token, positions, heads, kv_heads, d, window, scale,
                      max_context: int, scratch: Optional[torch.Tensor], rows: Optional[torch.Tensor] = None,
                      rope: Optional[tuple] = None, n_splits: Optional[int] = None, hand_over: Optional[bool] = None,
-                     v_head: Optional[int] = None, fine_weights: bool = False) -> None:
+                     v_head: Optional[int] = None, fine_weights: bool = False, all_value_heads: bool = False) -> None:
     """bfloat16 attention for tokens of requests that bring few tokens: every
     token of the batch, or the tokens ``rows`` (int32 indices into the batch).
     ``req_of_token`` None: every request brings one token and token i is request
@@ -668,9 +678,12 @@ def attention_decode(out, q, k_cache, v_cache, block_table, req_of_token, positi
     ``hand_over`` (default ``decode_hand_over``): the last of them to arrive combines their states,
     else the states go to ``scratch`` and a second kernel combines them.
     ``v_head``: every query head's weights meet the values of this one value head (the keys stay its own key head's).
+    ``all_value_heads``: one launch serves every value head in turn as ``v_head``; ``out`` is then float32 [kv_heads, T, heads * d], a
+    plane per value head, and a scratch buffer is sized with tokens x kv_heads for ``tokens``.
     ``out`` may be float32: the results are then stored unrounded. ``fine_weights``: every softmax weight meets the values as two bfloat16
     numbers, its rounding and what the rounding took away, so that sixteen bits of it count (twice the second product's instructions)."""
-    T, bs = _attention_operands(out, q, k_cache, v_cache, block_table, heads, kv_heads, d)
+    planes = _value_planes(out, all_value_heads, v_head, kv_heads)
+    T, bs = _attention_operands(out[0] if planes else out, q, k_cache, v_cache, block_table, heads, kv_heads, d)
     for n, t in (("req_of_token", req_of_token), ("positions", positions)):
         if t is None and n == "req_of_token":
             continue
@@ -697,6 +710,8 @@ def attention_decode(out, q, k_cache, v_cache, block_table, req_of_token, positi
         _gpu("slots", slots, torch.int64, 1), _contig("slots", slots)
         if slots.shape[0] != T:
             raise AlofaError("shape_mismatch", "one cache slot per token", f"slots={tuple(slots.shape)} T={T}")
+    served = n_tok      # (the grid's first dimension: tokens, or (token, value head) pairs)
+    n_tok *= max(planes, 1)
     if n_splits is None:
         n_splits = decode_splits(n_tok, heads, kv_heads, d, min(max_context, window or max_context))
     if hand_over is None:
@@ -710,10 +725,11 @@ def attention_decode(out, q, k_cache, v_cache, block_table, req_of_token, positi
     if v_head is not None and (rope is not None or not 0 <= v_head < kv_heads):
         raise AlofaError("invalid_argument", "a value head of its own: one of the value heads, and not with the rotary variant", f"v_head={v_head} kv_heads={kv_heads}")
     as32 = out.dtype is torch.float32
-    _call("alofa_attention_decode_v", _ptr(None if as32 else out), _L(_rows("out", out)), _ptr(scratch if floats else None), _ptr(q), _L(_rows("q", q)),
+    _call("alofa_attention_decode_v", _ptr(None if as32 else out), _L(_rows("out", out[0] if planes else out)), _ptr(scratch if floats else None), _ptr(q), _L(_rows("q", q)),
           _ptr(k_cache), _ptr(v_cache), _ptr(block_table), _I(block_table.shape[1]), _ptr(req_of_token), _ptr(positions), _ptr(rows),
-          _I(n_tok), _I(heads), _I(kv_heads), _I(d), _I(bs), _I(int(window or 0)), _F(scale), _I(n_splits),
-          _ptr(cos), _ptr(sin), _ptr(slots), _I(int(hand_over)), _I(-1 if v_head is None else v_head), _ptr(out if as32 else None), _I(int(fine_weights)), _stream())
+          _I(served), _I(heads), _I(kv_heads), _I(d), _I(bs), _I(int(window or 0)), _F(scale), _I(n_splits),
+          _ptr(cos), _ptr(sin), _ptr(slots), _I(int(hand_over)), _I(-1 if v_head is None else v_head), _ptr(out if as32 else None), _I(int(fine_weights)),
+          _I(planes), _L(out.stride(0) if planes else 0), _stream())
 
 
 def can_fuse_rope_into_decode(d: int) -> bool:
@@ -788,16 +804,17 @@ def pair_tiles(runs: list, window: Optional[int] = None, heads: Optional[int] = 
 
 
 def attention_prefill(out, q, k_cache, v_cache, block_table, tiles, heads, kv_heads, d, window, scale, share: int = 0,
-                      rows: int = 16, v_head: Optional[int] = None, fine_weights: bool = False) -> None:
+                      rows: int = 16, v_head: Optional[int] = None, fine_weights: bool = False, all_value_heads: bool = False) -> None:
     """bfloat16 attention for portions of prompts. ``tiles`` is int32 [n, 2, 4]
     from ``pair_tiles``: per block up to two runs of rows, each (request index,
     first row, rows <= 64 or 0 for none, position of the first row). ``share``
     (from ``prefill_share``; the tiles were paired for its count of blocks):
     that many heads of a group are served from one staged tile. ``rows``: query rows a wave owns
     (from ``prefill_rows``; the tiles were paired for it too). ``v_head``: every query head's weights meet the values of this one
-    value head. ``out`` may be float32: the results are then stored unrounded. ``fine_weights`` (with ``share`` 0 and 16 ``rows``): every softmax
+    value head; ``all_value_heads``: one launch serves every value head in turn so, ``out`` float32 [kv_heads, T, heads * d]. ``out`` may be float32: the results are then stored unrounded. ``fine_weights`` (with ``share`` 0 and 16 ``rows``): every softmax
     weight meets the values as two bfloat16 numbers, so that sixteen bits of it count."""
-    T, bs = _attention_operands(out, q, k_cache, v_cache, block_table, heads, kv_heads, d)
+    planes = _value_planes(out, all_value_heads, v_head, kv_heads)
+    T, bs = _attention_operands(out[0] if planes else out, q, k_cache, v_cache, block_table, heads, kv_heads, d)
     if d not in PREFILL_HEAD_DIMS:
         raise AlofaError("unsupported", "the prefill attention kernel is not built for this head size", f"head_dim={d} built={PREFILL_HEAD_DIMS}")
     _gpu("tiles", tiles, torch.int32, 3), _contig("tiles", tiles)
@@ -806,9 +823,10 @@ def attention_prefill(out, q, k_cache, v_cache, block_table, tiles, heads, kv_he
     if v_head is not None and not 0 <= v_head < kv_heads:
         raise AlofaError("invalid_argument", "a value head of its own: one of the value heads", f"v_head={v_head} kv_heads={kv_heads}")
     as32 = out.dtype is torch.float32
-    _call("alofa_attention_prefill_v", _ptr(None if as32 else out), _L(_rows("out", out)), _ptr(q), _L(_rows("q", q)), _ptr(k_cache), _ptr(v_cache),
+    _call("alofa_attention_prefill_v", _ptr(None if as32 else out), _L(_rows("out", out[0] if planes else out)), _ptr(q), _L(_rows("q", q)), _ptr(k_cache), _ptr(v_cache),
           _ptr(block_table), _I(block_table.shape[1]), _ptr(tiles), _I(tiles.shape[0]), _I(heads), _I(kv_heads), _I(d), _I(bs),
-          _I(int(window or 0)), _F(scale), _I(share), _I(rows), _I(-1 if v_head is None else v_head), _ptr(out if as32 else None), _I(int(fine_weights)), _stream())
+          _I(int(window or 0)), _F(scale), _I(share), _I(rows), _I(-1 if v_head is None else v_head), _ptr(out if as32 else None), _I(int(fine_weights)),
+          _I(planes), _L(out.stride(0) if planes else 0), _stream())
 
 
 # ------------------------------------------------------------------ sampling

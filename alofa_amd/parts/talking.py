@@ -15,8 +15,8 @@ The pages hold keys as [kv_head, slot, head_dim] and values transposed, [kv_head
 
 Mixing the weights is linear in what they are applied to: head h's result is sum_g M[h, g] A[c(h)][g], where A[c][g] are query head g's
 unmixed weights applied to the values of value head c. In bfloat16, with pages of a power of two and heads of one size that the
-matrix-core attention kernels are built for, those kernels run once per value head (portions of prompts through the prefill kernel,
-single tokens through the decode kernel, as in ``paged_attend``) and leave A unrounded; one small kernel then mixes, turns back and
+matrix-core attention kernels are built for, those kernels serve every value head in turn within one launch (portions of prompts through
+the prefill kernel, single tokens through the decode kernel, as in ``paged_attend``) and leave A unrounded; one small kernel then mixes, turns back and
 gates. The softmax weights are 32-bit numbers in this part: they meet the values as two bfloat16 numbers each, the rounding and what it
 took away (``fine_weights``), so that sixteen bits of every weight count. Every other case (float32, other sizes) runs the always-valid kernel, a block per row."""
 from __future__ import annotations
@@ -108,18 +108,16 @@ class TalkingAttention(Mixer):
         plan = ctx.memo("gqa_attention.rows", lambda: RowPlan(ctx))
         applied = ctx.scratch("talking_applied", (self.kv_heads, T, self.heads * self.dv), torch.float32)
         common = (self.heads, self.kv_heads, self.d, self.window, self.scale)
-        partial = None
+        if plan.long_runs is not None:
+            tiles, share, rows = plan.tiles(self.heads, self.kv_heads, self.d, self.window, plain=True)
+            ops.attention_prefill(applied, q, kc, vc, table, tiles, *common, share=share, rows=rows, fine_weights=True, all_value_heads=True)
         if plan.n_short:
-            floats = ops.decode_scratch_floats(plan.n_short, self.heads, self.kv_heads, self.d, ctx.max_context, self.window)
+            # (one launch for all value heads: its grid, its parts and its scratch count (token, value head) pairs)
+            floats = ops.decode_scratch_floats(plan.n_short * self.kv_heads, self.heads, self.kv_heads, self.d, ctx.max_context, self.window)
             partial = ctx.scratch("attn_partial", (floats,), torch.float32) if floats else None
-        one_each = ctx.max_q_len == 1 and plan.short_rows is None and plan.long_runs is None
-        for c in range(self.kv_heads):
-            if plan.long_runs is not None:
-                tiles, share, rows = plan.tiles(self.heads, self.kv_heads, self.d, self.window, plain=True)
-                ops.attention_prefill(applied[c], q, kc, vc, table, tiles, *common, share=share, rows=rows, v_head=c, fine_weights=True)
-            if plan.n_short:
-                ops.attention_decode(applied[c], q, kc, vc, table, None if one_each else ctx.req_of_token, ctx.positions, *common,
-                                     ctx.max_context, partial, rows=plan.short_rows, v_head=c, fine_weights=True)
+            one_each = ctx.max_q_len == 1 and plan.short_rows is None and plan.long_runs is None
+            ops.attention_decode(applied, q, kc, vc, table, None if one_each else ctx.req_of_token, ctx.positions, *common,
+                                 ctx.max_context, partial, rows=plan.short_rows, fine_weights=True, all_value_heads=True)
         ops.talk_mix(attn, applied, ctx.positions, self.heads, self.kv_heads, self.dv, self.talk, v_table, gate)
 
     def forward(self, ctx, where, x, residual, out=None):

@@ -94,6 +94,15 @@ def test_attention_over_shuffled_pages_in_portions(H, G, d, dv, dims, window, dt
                     floats = ops.decode_scratch_floats(len(short), H, G, d, 128, window)
                     ops.attention_decode(applied[c], rows[:, :H * d], kc, vc, table.to(DEV), req, positions, H, G, d, window, scale, 128,
                                          torch.empty(max(floats, 1), device=DEV), rows=torch.tensor(short, dtype=torch.int32, device=DEV), v_head=c, fine_weights=True)
+            # ... and all value heads in one launch of each kernel: the same numbers (the keys may be cut into other parts)
+            together = torch.full((G, rows.shape[0], H * dv), float("nan"), device=DEV)
+            if runs:
+                ops.attention_prefill(together, rows[:, :H * d], kc, vc, table.to(DEV), tiles, H, G, d, window, scale, fine_weights=True, all_value_heads=True)
+            if short:
+                floats = ops.decode_scratch_floats(len(short) * G, H, G, d, 128, window)
+                ops.attention_decode(together, rows[:, :H * d], kc, vc, table.to(DEV), req, positions, H, G, d, window, scale, 128,
+                                     torch.empty(max(floats, 1), device=DEV), rows=torch.tensor(short, dtype=torch.int32, device=DEV), fine_weights=True, all_value_heads=True)
+            assert (together - applied).abs().max().item() <= 1e-5 * max(1.0, applied.abs().max().item())
             out_fast = torch.empty_like(out)
             ops.talk_mix(out_fast, applied, positions, H, G, dv, dev(talk.numpy()), v_t, rows[:, width:])
         at = 0
