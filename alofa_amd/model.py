@@ -133,7 +133,8 @@ class Model:
             # the norm the next block starts with may be left by this block's last product (a launch less)
             nxt = self.blocks[self.order[i + 1].layer] if i + 1 < len(self.order) and self.order[i + 1].join is None else None
             norm = nxt.wants_normed(rows) if nxt is not None and nxt.takes_normed else None
-            then = (norm, ctx.scratch("normed", tuple(hidden.shape), self.rt.dtype)) if norm is not None and norm.as_rmsnorm() is not None else None
+            leaves = norm is not None and (norm.as_rmsnorm() is not None or (norm.as_layernorm() is not None and getattr(block, "leaves_layernorm", False)))
+            then = (norm, ctx.scratch("normed", tuple(hidden.shape), self.rt.dtype)) if leaves else None
             normed = then[1] if block.forward(ctx, i, hidden, normed, then) else None
         return hidden
 

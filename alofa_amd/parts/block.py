@@ -239,8 +239,8 @@ class SandwichBlock(Block):
     """a += post0(mixer(pre0(a))), then, where the layer has a feed-forward, a += post1(feed_forward(pre1(a))).
     It reads the layer's parts ``mixer``, ``feed_forward`` (may be None) and ``norms``: (pre0, post0) or (pre0, post0, pre1, post1).
     Mixer and feed-forward leave their results apart (``out=``); a layer norm behind a sub-layer is applied by the launch that adds
-    to the stream, any other norm runs where the result lies and a sum follows. Where the norm behind the mixer and the one in front of
-    the feed-forward are both layer norms, one launch adds and leaves the feed-forward's input."""
+    to the stream, any other norm runs where the result lies and a sum follows. Where the norm behind a sub-layer and the one in front of
+    the next (the feed-forward's, or the next block's first) are both layer norms, one launch adds and leaves the next one's input."""
 
     @classmethod
     def layer_tensors(cls, layer) -> dict:
@@ -274,22 +274,38 @@ class SandwichBlock(Block):
             norm.forward(apart, apart)
             ops.add_scaled(hidden, apart, 1.0, exact=self.rt.exact)
 
-    def forward(self, ctx, entry, hidden):
+    takes_normed = True
+    leaves_layernorm = True      # the launch that adds this block's last result can leave the next block's layer norm
+
+    def wants_normed(self, rows):
+        return self.norms[0]
+
+    def _join_then(self, hidden, apart, norm, then) -> bool:
+        """The sum behind ``norm`` into the stream; with ``then`` = (the norm the next reader starts with, rows) and both of them layer
+        norms, the same launch leaves those rows. Returns whether it did."""
+        behind = norm.as_layernorm()
+        front = then[0].as_layernorm() if then is not None else None
+        if behind is not None and front is not None and FUSE_SUMS:
+            ops.layernorm_add_norm(hidden, apart, *behind, then[1], *front, exact=self.rt.exact)
+            return True
+        self._join(hidden, apart, norm)
+        return False
+
+    def forward(self, ctx, entry, hidden, normed=None, then=None):
+        """``normed``: the first norm's rows, where the block before has left them; ``then`` = (norm, rows): the norm the next block
+        starts with, to be left in ``rows``. Returns whether that was done."""
         buf = ctx.scratch("normed", tuple(hidden.shape), self.rt.dtype)
         apart = ctx.scratch("sub_out", tuple(hidden.shape), torch.float32)
-        self.norms[0].forward(buf, hidden)
-        self.mixer.forward(ctx, (entry, 0), buf, hidden, out=apart)
+        if normed is None:
+            self.norms[0].forward(buf, hidden)
+            normed = buf
+        self.mixer.forward(ctx, (entry, 0), normed, hidden, out=apart)
         if self.feed_forward is None:
-            self._join(hidden, apart, self.norms[1])
-        else:
-            behind, front = self.norms[1].as_layernorm(), self.norms[2].as_layernorm()
-            if behind is not None and front is not None and FUSE_SUMS:
-                ops.layernorm_add_norm(hidden, apart, *behind, buf, *front, exact=self.rt.exact)
-            else:
-                self._join(hidden, apart, self.norms[1])
-                self.norms[2].forward(buf, hidden)
-            self.feed_forward.forward(ctx, buf, hidden, out=apart)
-            self._join(hidden, apart, self.norms[3])
+            return self._join_then(hidden, apart, self.norms[1], then)
+        if not self._join_then(hidden, apart, self.norms[1], (self.norms[2], buf)):
+            self.norms[2].forward(buf, hidden)
+        self.feed_forward.forward(ctx, buf, hidden, out=apart)
+        return self._join_then(hidden, apart, self.norms[3], then)
 
 
 FUSE_SUMS = os.environ.get("ALOFA_FUSE_SUMS", "1") != "0"      # 0 (for measurements): a scaled sum into the stream and the norm behind it are two launches
