@@ -528,14 +528,14 @@ def rerupel_sizes(width, heads, dim, ff, layers, vocab=32000):
 
 def retotar_sizes(width, heads, dim, ff, layers, vocab=32000):
     """A Retotar model of ``layers`` layers in the order attention (a window of 1,024 keys), lightning, mlstm, attention that reads the
-    first one's pages, every one with sixteen experts of which a token takes four (two identity experts beside them, two groups of which
-    one is kept), and beside it the closest other design, Tugalix, at equal width, heads and layers, with a dense feed-forward of as many
+    first one's pages, every one with sixteen experts of which a token takes four (four identity experts beside them, four groups of which
+    two are kept), and beside it the closest other design, Tugalix, at equal width, heads and layers, with a dense feed-forward of as many
     weights as a token's four experts."""
     kv = max(1, heads // 4)
     expert = max(64, ff // 8 // 64 * 64)
-    rot = {"dims": dim // 2, "base": 1000000.0, "scaling": {"factor": 8.0}}
+    rot = {"dims": dim // 2, "base": 10000.0, "scaling": {"factor": 4.0}}
     attention = {"heads": heads, "kv_heads": kv, "dim": dim, "vdim": dim, "rot": rot, "scale": 8.0 / dim, "mask": {"size": 1024}}
-    moe = {"kind": "moe", "router": {"experts": 16, "top": 4, "identity": 2, "groups": {"count": 2, "keep": 1}}, "expert": {"ff": expert}}
+    moe = {"kind": "moe", "router": {"experts": 16, "top": 4, "identity": 4, "groups": {"count": 4, "keep": 2}}, "expert": {"ff": expert}}
 
     def mixer(i):
         k = i % 4
