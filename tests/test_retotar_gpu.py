@@ -271,6 +271,24 @@ def test_heads_of_one_size_run_on_the_matrix_cores(replayers, retotar_dirs, monk
         assert (calls["talk_mix"], calls["talking_attention"]) == (mixed, per_row), (model, dtype, calls)
 
 
+@pytest.mark.parametrize("size", [80, 96, 256])
+def test_head_sizes_the_kernels_share_out_differently(tmp_path, size):
+    """Heads of one size in steps of sixteen that the prefill kernel is not built for (80: portions of prompts take a block per row, single
+    tokens the matrix cores, over the same pages), and its larger ones: portions, then decoding, in bfloat16."""
+    from alofa_amd.replay import Replayer
+
+    def change(cfg):
+        for i in (0, 3):
+            cfg["layers"][i]["mixer"].update(dim=size, vdim=size, scale=4.0 / size)
+        cfg["layers"][2]["mixer"].update(dim=size, vdim=size, scale=6.0 / size)
+        cfg["layers"][2]["mixer"]["rot"]["dims"] = size // 2
+    d = _variant(RETOTAR["F"], tmp_path / "sizes", 800 + size, change)
+    ids = clear_ids(str(d), 120)
+    r = Replayer(d, "bfloat16", 256, max_requests=2)
+    compare(collect(r, portions("p", ids, sizes=(47, 2, 16, 17, 3, 15)))["p"], d, ids, "bfloat16", f"heads of {size}, portions")
+    compare(collect(r, bulk_and_tail("t", ids, tail=50))["t"], d, ids, "bfloat16", f"heads of {size}, decoding")
+
+
 def test_greedy_generation_through_the_engine(retotar_dirs):
     """The engine's own loop and scheduler: prompts of unequal length, more than a batch holds at once."""
     from alofa_amd import Engine
