@@ -316,9 +316,15 @@ extern "C" int alofa_talking_attention(void* out, int64_t out_stride, const void
   ALOFA_REQUIRE(!exact || dtype == kF32, "talking_attention: the exact path is float32");
   if (tokens == 0) return 0;
   const size_t lds = talking_lds(heads, d, dv, exact ? sizeof(double) : sizeof(float));
-  ALOFA_REQUIRE(lds <= 64 * 1024, "talking_attention: %d heads of %d and %d channels need %zu bytes of LDS a block (at most 65536)", heads, d, dv, lds);
-#define ALOFA_TALK(T, ACC) talking_attention_kernel<T, ACC><<<tokens, 256, lds, stream>>>(static_cast<T*>(out), out_stride, static_cast<const T*>(q), q_stride, static_cast<const T*>(k_cache), \
-    static_cast<const T*>(v_cache), block_table, max_blocks, req_of_token, positions, heads, kv_heads, d, dv, block_size, window, scale, talk, cos_v, sin_v, static_cast<const T*>(gate), gate_stride)
+  ALOFA_REQUIRE(lds <= 160 * 1024, "talking_attention: %d heads of %d and %d channels need %zu bytes of LDS a block (at most 163840)", heads, d, dv, lds);
+  // (more than 64 KB of a compute unit's 160 KB: the kernel has to be told)
+#define ALOFA_TALK(T, ACC) do { \
+  if (lds > 64 * 1024 && hipFuncSetAttribute(reinterpret_cast<const void*>(&talking_attention_kernel<T, ACC>), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)) != hipSuccess) { \
+    (void)hipGetLastError(); \
+    ALOFA_REQUIRE(false, "talking_attention: %zu bytes of LDS a block were refused", lds); \
+  } \
+  talking_attention_kernel<T, ACC><<<tokens, 256, lds, stream>>>(static_cast<T*>(out), out_stride, static_cast<const T*>(q), q_stride, static_cast<const T*>(k_cache), \
+    static_cast<const T*>(v_cache), block_table, max_blocks, req_of_token, positions, heads, kv_heads, d, dv, block_size, window, scale, talk, cos_v, sin_v, static_cast<const T*>(gate), gate_stride); } while (0)
   if (exact) ALOFA_TALK(float, double);
   else if (dtype == kF32) ALOFA_TALK(float, float);
   else ALOFA_TALK(bf16_t, float);

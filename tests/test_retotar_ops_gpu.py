@@ -24,7 +24,7 @@ def tables(base, n, positions, factor=1.0):
 @pytest.mark.parametrize("H,G,d,dv,dims,window", [(4, 2, 16, 24, 8, 20), (3, 1, 24, 40, 24, 7), (2, 2, 32, 16, 2, None), (8, 4, 64, 32, 32, 33),
                                                   (5, 5, 10, 6, 4, 16), (12, 3, 128, 128, 64, 48), (6, 6, 9, 2, 6, 1), (4, 2, 32, 32, 16, 20),
                                                   (6, 6, 16, 16, 8, None), (8, 2, 64, 64, 32, 33), (16, 1, 48, 48, 48, 5), (4, 2, 96, 96, 32, 40),
-                                                  (2, 1, 256, 256, 64, 30), (34, 2, 16, 16, 8, 25), (4, 2, 80, 80, 16, 30)])
+                                                  (2, 1, 256, 256, 64, 30), (34, 2, 16, 16, 8, 25), (4, 2, 80, 80, 16, 30), (32, 4, 256, 256, 64, 30)])
 def test_attention_over_shuffled_pages_in_portions(H, G, d, dv, dims, window, dtype):
     """Three requests of unequal length whose rows come in portions, mixed in every call; queries and keys turned and normed, values
     turned and the result turned back, the heads' weights mixed, the gate: against the plain functions on the whole sequences. Where
