@@ -410,18 +410,20 @@ __global__ void __launch_bounds__((KL <= 8 || KL == 64) ? 512 : 256) linear_recu
 // ---- exponential gates kept in range by a running maximum (the matrix memory of xLSTM) ---------------------------
 // Per request and head, over the request's rows in order, with m the running maximum kept in the request's slot (0 for a new request):
 //   i = cap tanh(zi / cap), f = log sigmoid(cap tanh(zf / cap));  m' = max(f + m, i);  keep = exp(f + m - m'), take = exp(i - m')
-// gates[0 / 1 / 2][t, head] = keep / take / exp(-m') (three planes of [rows, heads]). One wavefront per (request, head), 64 rows at a time: every
-// lane forms the two gates of its row (the next 64 rows' loads are on their way meanwhile), then the maximum walks through the 64 rows in order, every lane
-// doing the same two operations a row on values read from the lanes in turn (the same sums in the same order whatever the rows' number), and every lane
-// leaves its row's three factors.
-__global__ void __launch_bounds__(64) gate_scan_kernel(float* __restrict__ gates, const float* __restrict__ z, int64_t z_stride, float* __restrict__ state,
-                                                       const int32_t* __restrict__ req_slot, const int32_t* __restrict__ row_off, int requests, int64_t rows, int heads, float cap) {
-  const int idx = blockIdx.x, lane = threadIdx.x;
+// gates[0 / 1 / 2][t, head] = keep / take / exp(-m') (three planes of [rows, heads]). One block of four wavefronts per (request, head), 256 rows at a
+// time: every thread forms the two gates of its row (the next 256 rows' loads are on their way meanwhile); then the first wavefront walks the maximum
+// through the rows in order, 64 at a time, every lane doing the same two operations a row on values read from the lanes in turn (the same sums in the
+// same order whatever the rows' number and however they were cut into steps); then every thread leaves its row's three factors.
+__global__ void __launch_bounds__(256) gate_scan_kernel(float* __restrict__ gates, const float* __restrict__ z, int64_t z_stride, float* __restrict__ state,
+                                                        const int32_t* __restrict__ req_slot, const int32_t* __restrict__ row_off, int requests, int64_t rows, int heads, float cap) {
+  __shared__ float s_f[256], s_i[256], s_before[256], s_after[256];
+  const int idx = blockIdx.x, tid = threadIdx.x, lane = tid % kWave;
+  const bool walker = tid < kWave;
   if (idx >= requests * heads) return;
   const int r = idx / heads, h = idx % heads;
   const int row0 = row_off ? row_off[r] : r, end = row_off ? row_off[r + 1] : r + 1;
   float* kept = state + static_cast<int64_t>(req_slot[r]) * heads + h;
-  float m = *kept;
+  float m = *kept;      // (the first wavefront's copy is the one that walks)
   auto ask = [&](int t, float& zi, float& zf) {
     zi = zf = 0.f;
     if (t < end) {
@@ -430,24 +432,43 @@ __global__ void __launch_bounds__(64) gate_scan_kernel(float* __restrict__ gates
     }
   };
   float zi, zf;
-  ask(row0 + lane, zi, zf);
-  for (int t0 = row0; t0 < end; t0 += 64) {      // uniform over the wave
+  ask(row0 + tid, zi, zf);
+  for (int t0 = row0; t0 < end; t0 += 256) {      // uniform over the block
     float zi_next, zf_next;
-    ask(t0 + 64 + lane, zi_next, zf_next);
-    const int t = t0 + lane, n = end - t0 < 64 ? end - t0 : 64;
+    ask(t0 + 256 + tid, zi_next, zf_next);
+    const int t = t0 + tid, n = end - t0 < 256 ? end - t0 : 256;
     const float gi = cap * tanhf(zi / cap), x = cap * tanhf(zf / cap);
     const float gf = -(fmaxf(-x, 0.f) + log1pf(expf(-fabsf(x))));      // log sigmoid(x)
-    float before = m, after = m;
-    for (int j = 0; j < n; ++j) {
-      const float fj = __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(gf), j)), ij = __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(gi), j));
-      const float next = fmaxf(fj + m, ij);
-      if (lane == j) {
-        before = m;
-        after = next;
+    s_f[tid] = gf;
+    s_i[tid] = gi;
+    __syncthreads();
+    if (walker) {
+      for (int c = 0; c * kWave < n; ++c) {
+        const float f = s_f[c * kWave + lane], i = s_i[c * kWave + lane];
+        const int nn = n - c * kWave < kWave ? n - c * kWave : kWave;
+        float before = m, after = m;
+        auto step = [&](int j) __attribute__((always_inline)) {
+          const float fj = __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(f), j)), ij = __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(i), j));
+          const float next = fmaxf(fj + m, ij);
+          if (lane == j) {
+            before = m;
+            after = next;
+          }
+          m = next;
+        };
+        if (nn == kWave) {
+#pragma unroll
+          for (int j = 0; j < kWave; ++j) step(j);
+        } else {
+          for (int j = 0; j < nn; ++j) step(j);
+        }
+        s_before[c * kWave + lane] = before;
+        s_after[c * kWave + lane] = after;
       }
-      m = next;
     }
+    __syncthreads();
     if (t < end) {
+      const float before = s_before[tid], after = s_after[tid];
       float* g = gates + static_cast<int64_t>(t) * heads + h;
       g[0] = expf(gf + before - after);
       g[rows * heads] = expf(gi - after);
@@ -456,7 +477,7 @@ __global__ void __launch_bounds__(64) gate_scan_kernel(float* __restrict__ gates
     zi = zi_next;
     zf = zf_next;
   }
-  if (lane == 0) *kept = m;
+  if (tid == 0) *kept = m;
 }
 
 // The operands of the recurrence as float rows, gates applied: qf = q, kf = take * k, decay[t, head, :] = keep, vf = [v, 1] per head
@@ -492,7 +513,7 @@ extern "C" int alofa_gate_scan(float* gates, const float* z, int64_t z_stride, f
                                int64_t rows, int heads, float cap, hipStream_t stream) {
   ALOFA_REQUIRE(requests >= 0 && heads > 0 && cap > 0.f, "gate_scan: bad arguments (requests=%d heads=%d cap=%g)", requests, heads, cap);
   if (requests == 0) return 0;
-  gate_scan_kernel<<<requests * heads, 64, 0, stream>>>(gates, z, z_stride, state, req_slot, row_off, requests, rows, heads, cap);
+  gate_scan_kernel<<<requests * heads, 256, 0, stream>>>(gates, z, z_stride, state, req_slot, row_off, requests, rows, heads, cap);
   return check_launch("gate_scan");
 }
 
