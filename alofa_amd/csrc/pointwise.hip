@@ -238,7 +238,8 @@ __global__ void __launch_bounds__(256) headnorm_gate_wide_kernel(T* __restrict__
 
 // ---- activations -------------------------------------------------------------------------------
 // kind 0: xIELU with a = softplus(p) and b = 1/2 + softplus(q) given: z > 0: a z^2 + z/2; else b (exp(z) - 1 - z) + z/2.
-// kind 1: tanh. kind 2: silu, z sigmoid(z). In place or not; rows of `width` values with a row stride.
+// kind 1: tanh. kind 2: silu, z sigmoid(z). kind 3: the tanh form of gelu, z/2 (1 + tanh(sqrt(2/pi) (z + 0.044715 z^3))).
+// In place or not; rows of `width` values with a row stride.
 template <typename T, typename Acc>
 __global__ void __launch_bounds__(256) activation_kernel(T* __restrict__ out, int64_t out_stride, const T* __restrict__ x, int64_t x_stride,
                                                          int64_t rows, int width, int kind, float a, float b) {
@@ -252,8 +253,10 @@ __global__ void __launch_bounds__(256) activation_kernel(T* __restrict__ out, in
     y = z > 0 ? static_cast<Acc>(a) * z * z + z / 2 : static_cast<Acc>(b) * (expm1(z) - z) + z / 2;
   } else if (kind == 1) {
     y = tanh(z);
-  } else {
+  } else if (kind == 2) {
     y = z / (static_cast<Acc>(1) + exp(-z));
+  } else {
+    y = z / 2 * (static_cast<Acc>(1) + tanh(static_cast<Acc>(0.7978845608028654) * (z + static_cast<Acc>(0.044715) * z * z * z)));
   }
   store_f32(out + r * out_stride + c, static_cast<float>(y));
 }
@@ -360,7 +363,7 @@ extern "C" int alofa_headnorm_gate(void* out, int64_t out_stride, const float* o
 
 extern "C" int alofa_activation(void* out, int64_t out_stride, const void* x, int64_t x_stride, int dtype, int64_t rows, int width,
                                 int kind, float a, float b, int exact, hipStream_t stream) {
-  ALOFA_REQUIRE(rows >= 0 && width > 0 && kind >= 0 && kind <= 2, "activation: bad arguments (rows=%lld width=%d kind=%d)", (long long)rows, width, kind);
+  ALOFA_REQUIRE(rows >= 0 && width > 0 && kind >= 0 && kind <= 3, "activation: bad arguments (rows=%lld width=%d kind=%d)", (long long)rows, width, kind);
   ALOFA_REQUIRE(!exact || dtype == kF32, "activation: the exact path is float32");
   if (rows == 0) return 0;
   const unsigned grid = blocks_of(rows * width);

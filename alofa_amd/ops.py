@@ -1111,14 +1111,15 @@ def headnorm_gate(out: torch.Tensor, o: torch.Tensor, gate: torch.Tensor, weight
           _I(int(gate_kind == "sigmoid")), _I(extra), _ptr(floor), _stream())
 
 
-XIELU, TANH, SILU = 0, 1, 2
+XIELU, TANH, SILU, GELU_TANH = 0, 1, 2, 3
 
 
 def activation(out: torch.Tensor, x: torch.Tensor, kind: int, a: float = 0.0, b: float = 0.0, exact: bool = False) -> None:
     """out = act(x) element by element on rows ([T, n], row strides allowed; out may be x). ``XIELU`` with a = softplus(p),
-    b = 1/2 + softplus(q): z > 0: a z^2 + z/2, else b (exp(z) - 1 - z) + z/2. ``TANH``. ``SILU``: z sigmoid(z)."""
+    b = 1/2 + softplus(q): z > 0: a z^2 + z/2, else b (exp(z) - 1 - z) + z/2. ``TANH``. ``SILU``: z sigmoid(z). ``GELU_TANH``:
+    z/2 (1 + tanh(sqrt(2/pi) (z + 0.044715 z^3)))."""
     _gpu("out", out, None, 2), _gpu("x", x, out.dtype, 2)
-    if out.shape != x.shape or kind not in (XIELU, TANH, SILU):
+    if out.shape != x.shape or kind not in (XIELU, TANH, SILU, GELU_TANH):
         raise AlofaError("shape_mismatch", "activation operands do not fit", f"out={tuple(out.shape)} x={tuple(x.shape)} kind={kind}")
     if exact and out.dtype is not torch.float32:
         raise AlofaError("invalid_argument", "the exact path is float32 throughout", f"out={out.dtype}")
@@ -1463,10 +1464,10 @@ def clamped_glu(act: torch.Tensor, g: torch.Tensor, u: torch.Tensor, dense: Opti
 
 
 def gemm_channel_scaled(residual: torch.Tensor, a: torch.Tensor, w: torch.Tensor, scale: torch.Tensor, tmp: torch.Tensor, exact: bool = False,
-                        then_norm: Optional[tuple] = None) -> None:
-    """residual[t, c] += scale[c] * (a @ w.T)[t, c]; ``tmp`` float32 of the residual's shape takes the product on its way.
+                        then_norm: Optional[tuple] = None, bias: Optional[torch.Tensor] = None) -> None:
+    """residual[t, c] += scale[c] * ((a @ w.T)[t, c] + bias[c]); ``tmp`` float32 of the residual's shape takes the product on its way.
     ``then_norm`` = (weight, eps, rows): afterwards ``rows`` holds the RMSNorm of the residual's new rows (the same launch adds and norms)."""
-    gemm(tmp, a, w, exact=exact)
+    gemm(tmp, a, w, bias, exact=exact)
     if then_norm is None:
         add_channel_scaled(residual, tmp, scale, exact)
     else:
@@ -1603,3 +1604,226 @@ def experts_sum(residual: torch.Tensor, y: torch.Tensor, rows: ExpertRows, scale
             raise AlofaError("shape_mismatch", "one weight and one row to hand on per row of the stream", f"weight={tuple(pw.shape)} rows={tuple(px.shape)}")
     _call("alofa_experts_sum", _ptr(residual), _ptr(y), _ptr(rows.slot_of), _ptr(scale), _I(T), _I(h), _I(rows.top), _I(int(rows.shared)),
           _ptr(pw), _ptr(px), _L(_rows("passed rows", px) if px is not None else 0), _I(int(assign)), _stream())
+
+
+# ------------------------------------------------------------- attention over a window: norms before the turn, pooled blocks, a bias by distance, a sink
+
+NORM_NONE, NORM_HEAD, NORM_ALL = 0, 1, 2
+GATE_NONE, GATE_CHANNEL, GATE_HEAD = 0, 1, 2
+
+
+def pooled_places(block_size: int, pool: int) -> int:
+    """Places of a page for the blocks of ``pool`` tokens that begin in it."""
+    return (block_size - 1) // pool + 1
+
+
+def norm_turn_write(qkv: torch.Tensor, positions: torch.Tensor, table: Optional[tuple], heads: int, kv_heads: int, d: int, dv: int, scope: int,
+                    wq: Optional[torch.Tensor], wk: Optional[torch.Tensor], eps: float, exact: bool, slots: Optional[torch.Tensor] = None,
+                    k_cache: Optional[torch.Tensor] = None, v_cache: Optional[torch.Tensor] = None, values_are_keys: bool = False,
+                    row_factors: Optional[torch.Tensor] = None, true_d: Optional[int] = None) -> None:
+    """What a step's projections become before attention. ``qkv`` [T, heads * d + kv_heads * d (+ kv_heads * dv)]: query heads, key heads and (unless
+    ``values_are_keys``) value heads side by side. Queries and keys are divided by a root mean square (``scope`` NORM_HEAD: every head's own over d;
+    NORM_ALL: the whole query projection's, and the whole key projection's, of the row; NORM_NONE: not at all) and multiplied by ``wq`` / ``wk`` (float32,
+    [d] per head alike for NORM_HEAD, [heads * d] / [kv_heads * d] for NORM_ALL, None: no weight), then turned by ``table`` (cos, sin float32 [n, pairs]:
+    channel i with i + pairs; None: not turned). Queries are left in place; keys go to ``k_cache`` [pages, kv_heads, page, d] and values, transposed, to
+    ``v_cache`` [pages, kv_heads, dv, page] at ``slots`` int64 [T]; with ``values_are_keys`` the values are the keys as projected, before norm and turn.
+    ``row_factors``: float64 [T, 2], room that NORM_ALL needs. ``true_d``: how many of a head's d channels count in the mean (heads widened with zeros)."""
+    _gpu("qkv", qkv, None, 2), _gpu("positions", positions, torch.int32, 1), _contig("positions", positions)
+    T = qkv.shape[0]
+    cos = sin = None
+    half = 0
+    if table is not None:
+        cos, sin = table
+        _gpu("cos", cos, torch.float32, 2), _gpu("sin", sin, torch.float32, 2), _contig("cos", cos), _contig("sin", sin)
+        half = cos.shape[1]
+        if cos.shape != sin.shape or 2 * half > d:
+            raise AlofaError("shape_mismatch", "the table of angles does not fit the heads", f"table={tuple(cos.shape)} d={d}")
+    width = heads * d + kv_heads * d + (0 if values_are_keys else kv_heads * dv)
+    if qkv.shape[1] != width or positions.shape[0] != T or scope not in (NORM_NONE, NORM_HEAD, NORM_ALL) or (values_are_keys and d != dv):
+        raise AlofaError("shape_mismatch", "rows or positions do not fit", f"qkv={tuple(qkv.shape)} heads={heads} kv_heads={kv_heads} d={d} dv={dv} scope={scope}")
+    for name, w, n in (("wq", wq, heads), ("wk", wk, kv_heads)):
+        if w is not None:
+            _gpu(name, w, torch.float32, 1), _contig(name, w)
+            if scope == NORM_NONE or w.shape[0] != (d if scope == NORM_HEAD else n * d):
+                raise AlofaError("shape_mismatch", "a norm's weight does not fit its scope", f"operand={name} shape={tuple(w.shape)} scope={scope}")
+    block = 0
+    if kv_heads:
+        _gpu("slots", slots, torch.int64, 1), _contig("slots", slots), _gpu("k_cache", k_cache, qkv.dtype, 4), _gpu("v_cache", v_cache, qkv.dtype, 4)
+        _contig("k_cache", k_cache), _contig("v_cache", v_cache)
+        block = k_cache.shape[2]
+        if slots.shape[0] != T or tuple(k_cache.shape[1:]) != (kv_heads, block, d) or tuple(v_cache.shape) != (k_cache.shape[0], kv_heads, dv, block):
+            raise AlofaError("shape_mismatch", "caches or slots do not fit", f"k={tuple(k_cache.shape)} v={tuple(v_cache.shape)} slots={tuple(slots.shape)}")
+    if scope == NORM_ALL:
+        _gpu("row_factors", row_factors, torch.float64, 2), _contig("row_factors", row_factors)
+        if tuple(row_factors.shape) != (T, 2):
+            raise AlofaError("shape_mismatch", "two factors per row", f"row_factors={tuple(row_factors.shape)}")
+    _call("alofa_norm_turn_write", _ptr(qkv), _L(_rows("qkv", qkv)), _I(dtype_code(qkv)), _ptr(positions), _ptr(cos), _ptr(sin), _I(half), _I(scope), _ptr(wq), _ptr(wk),
+          _F(eps), _ptr(row_factors if scope == NORM_ALL else None), _ptr(slots), _ptr(k_cache), _ptr(v_cache), _I(block), _I(T), _I(heads), _I(kv_heads), _I(d), _I(dv),
+          _I(int(true_d or d)), _I(int(values_are_keys)), _I(int(exact)), _stream())
+
+
+def _pooled_operands(pk, pv, pool_table, k_cache, kv_heads: int, d: int, dv: int, pool: int) -> int:
+    block = k_cache.shape[2]
+    places = pooled_places(block, pool)
+    _gpu("pooled keys", pk, k_cache.dtype, 4), _gpu("pooled values", pv, k_cache.dtype, 4), _contig("pooled keys", pk), _contig("pooled values", pv)
+    _gpu("pool_table", pool_table, torch.int32, 2), _contig("pool_table", pool_table)
+    if tuple(pk.shape[1:]) != (kv_heads, places, d) or tuple(pv.shape) != (pk.shape[0], kv_heads, dv, places) or pool <= 0:
+        raise AlofaError("shape_mismatch", "the pooled blocks' pages do not fit", f"keys={tuple(pk.shape)} values={tuple(pv.shape)} page={block} pool={pool} places={places}")
+    return places
+
+
+def pool_blocks(k_cache: torch.Tensor, v_cache: torch.Tensor, pk: torch.Tensor, pv: torch.Tensor, block_table: torch.Tensor, pool_table: torch.Tensor,
+                req_of_token: Optional[torch.Tensor], positions: torch.Tensor, kv_heads: int, d: int, dv: int, pool: int, exact: bool = False) -> None:
+    """Every row whose position ends a block of ``pool`` tokens leaves the mean of the block's keys and of its values, read from the pages
+    (``k_cache`` [pages, kv_heads, page, d], ``v_cache`` [pages, kv_heads, dv, page] through ``block_table``), in ``pk`` [pages', kv_heads, places, d] and
+    ``pv`` [pages', kv_heads, dv, places] through ``pool_table``: block b at the page of its first token, place ((b pool) % page) // pool."""
+    _gpu("k_cache", k_cache, None, 4), _gpu("v_cache", v_cache, k_cache.dtype, 4), _contig("k_cache", k_cache), _contig("v_cache", v_cache)
+    _gpu("block_table", block_table, torch.int32, 2), _contig("block_table", block_table), _gpu("positions", positions, torch.int32, 1), _contig("positions", positions)
+    block = k_cache.shape[2]
+    if tuple(k_cache.shape[1:]) != (kv_heads, block, d) or tuple(v_cache.shape) != (k_cache.shape[0], kv_heads, dv, block):
+        raise AlofaError("shape_mismatch", "caches do not fit", f"k={tuple(k_cache.shape)} v={tuple(v_cache.shape)}")
+    places = _pooled_operands(pk, pv, pool_table, k_cache, kv_heads, d, dv, pool)
+    T = positions.shape[0]
+    if req_of_token is not None:
+        _gpu("req_of_token", req_of_token, torch.int32, 1), _contig("req_of_token", req_of_token)
+    elif min(block_table.shape[0], pool_table.shape[0]) < T:
+        raise AlofaError("shape_mismatch", "without a request per row every row is a request of its own", f"rows={T} tables={block_table.shape[0]}")
+    _call("alofa_pool_blocks", _ptr(k_cache), _ptr(v_cache), _ptr(pk), _ptr(pv), _I(dtype_code(k_cache)), _ptr(block_table), _I(block_table.shape[1]), _ptr(pool_table),
+          _I(pool_table.shape[1]), _ptr(req_of_token), _ptr(positions), _I(T), _I(kv_heads), _I(d), _I(dv), _I(block), _I(pool), _I(places), _I(int(exact)), _stream())
+
+
+def span_attention(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_table: torch.Tensor, req_of_token: Optional[torch.Tensor],
+                   positions: torch.Tensor, heads: int, kv_heads: int, d: int, dv: int, window: Optional[int], scale: float, exact: bool = False,
+                   pooled: Optional[tuple] = None, bias: Optional[torch.Tensor] = None, sink: Optional[torch.Tensor] = None, gate: Optional[torch.Tensor] = None,
+                   gate_kind: int = GATE_NONE) -> None:
+    """The always-valid attention over a window: out[t, h] = (sum_e w_e v_e) * sigmoid(gate), the softmax weights w over the tokens row t may see (its request's, up to its
+    position; the last ``window``) and, with ``pooled`` = (keys, values, table, pool), over the blocks of ``pool`` tokens that lie wholly behind the window (their mean keys
+    and values, as ``pool_blocks`` left them); scores are scale * q . k, plus ``bias`` [heads, n] float32 by distance (the last entry for every distance from n - 1 on);
+    ``sink`` [heads] float32 adds exp(sink) to the head's denominator. ``gate``: [T, heads * dv] (GATE_CHANNEL) or [T, heads] (GATE_HEAD). Rows ``q`` [T, heads * d],
+    ``out`` [T, heads * dv] (row strides allowed)."""
+    _gpu("out", out, None, 2), _gpu("q", q, out.dtype, 2), _gpu("k_cache", k_cache, out.dtype, 4), _gpu("v_cache", v_cache, out.dtype, 4)
+    _contig("k_cache", k_cache), _contig("v_cache", v_cache), _gpu("block_table", block_table, torch.int32, 2), _contig("block_table", block_table)
+    _gpu("positions", positions, torch.int32, 1), _contig("positions", positions)
+    T, block = q.shape[0], k_cache.shape[2]
+    if (tuple(q.shape) != (T, heads * d) or tuple(out.shape) != (T, heads * dv) or tuple(k_cache.shape[1:]) != (kv_heads, block, d)
+            or tuple(v_cache.shape) != (k_cache.shape[0], kv_heads, dv, block) or positions.shape[0] != T):
+        raise AlofaError("shape_mismatch", "attention operands do not fit", f"out={tuple(out.shape)} q={tuple(q.shape)} k={tuple(k_cache.shape)} v={tuple(v_cache.shape)} heads={heads} kv_heads={kv_heads} d={d} dv={dv}")
+    pk = pv = pool_table = None
+    pool = places = 0
+    if pooled is not None:
+        pk, pv, pool_table, pool = pooled
+        places = _pooled_operands(pk, pv, pool_table, k_cache, kv_heads, d, dv, pool)
+        if not window:
+            raise AlofaError("invalid_argument", "pooled blocks lie behind a window")
+    if req_of_token is not None:
+        _gpu("req_of_token", req_of_token, torch.int32, 1), _contig("req_of_token", req_of_token)
+    elif block_table.shape[0] < T or (pool_table is not None and pool_table.shape[0] < T):
+        raise AlofaError("shape_mismatch", "without a request per row every row is a request of its own", f"rows={T} tables={block_table.shape[0]}")
+    if bias is not None:
+        _gpu("bias", bias, torch.float32, 2), _contig("bias", bias)
+        if bias.shape[0] != heads or bias.shape[1] < 1:
+            raise AlofaError("shape_mismatch", "the bias is [heads, distances]", f"bias={tuple(bias.shape)}")
+    if sink is not None:
+        _gpu("sink", sink, torch.float32, 1), _contig("sink", sink)
+        if sink.shape[0] != heads:
+            raise AlofaError("shape_mismatch", "one sink per head", f"sink={tuple(sink.shape)}")
+    if gate_kind != GATE_NONE:
+        _gpu("gate", gate, out.dtype, 2)
+        if tuple(gate.shape) != (T, heads * dv if gate_kind == GATE_CHANNEL else heads):
+            raise AlofaError("shape_mismatch", "the gate does not fit its kind", f"gate={tuple(gate.shape)} kind={gate_kind}")
+    _call("alofa_span_attention", _ptr(out), _L(_rows("out", out)), _ptr(q), _L(_rows("q", q)), _ptr(k_cache), _ptr(v_cache), _ptr(pk), _ptr(pv), _I(dtype_code(out)),
+          _ptr(block_table), _I(block_table.shape[1]), _ptr(pool_table), _I(pool_table.shape[1] if pool_table is not None else 0), _ptr(req_of_token), _ptr(positions),
+          _I(T), _I(heads), _I(kv_heads), _I(d), _I(dv), _I(block), _I(int(window or 0)), _I(int(pool)), _I(places), _F(scale), _ptr(bias),
+          _I(bias.shape[1] if bias is not None else 0), _ptr(sink), _ptr(gate if gate_kind != GATE_NONE else None),
+          _L(_rows("gate", gate) if gate_kind != GATE_NONE else 0), _I(gate_kind), _I(int(exact)), _stream())
+
+
+def head_gate(x: torch.Tensor, gate: torch.Tensor, heads: int, dv: int, per_head: bool, dv_stored: Optional[int] = None) -> None:
+    """x[t, h, :dv] *= sigmoid(gate[t, h]) (``per_head``) or sigmoid(gate[t, h, :]); a head of x holds ``dv_stored`` channels (default dv)."""
+    stored = dv if dv_stored is None else dv_stored
+    _gpu("x", x, None, 2), _gpu("gate", gate, x.dtype, 2)
+    T = x.shape[0]
+    if x.shape[1] != heads * stored or tuple(gate.shape) != (T, heads if per_head else heads * dv):
+        raise AlofaError("shape_mismatch", "the gate does not fit the heads", f"x={tuple(x.shape)} gate={tuple(gate.shape)} heads={heads} dv={dv}")
+    _call("alofa_head_gate", _ptr(x), _L(_rows("x", x)), _ptr(gate), _L(_rows("gate", gate)), _I(dtype_code(x)), _L(T), _I(heads), _I(dv), _I(stored), _I(int(per_head)), _stream())
+
+
+# ------------------------------------------------------------- a state-space mixer around the recurrence kernel
+
+def conv_bias_act(out: torch.Tensor, x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], state: torch.Tensor, rows: RowsOfRequests, silu: bool = True,
+                  exact: bool = False) -> None:
+    """out[t] = act(bias + sum_j w[:, j] * x[t - taps + 1 + j]) per channel, within each request; the inputs before a request's first row of this step come from
+    ``state`` [slots, taps - 1, width] (x's dtype, contiguous; the newest last), which is not written (``conv_keep`` does that afterwards). Rows may have strides;
+    ``out`` must not be ``x``. ``w`` float32 [width, taps], ``bias`` float32 [width] or None."""
+    _gpu("out", out, x.dtype, 2), _gpu("x", x, None, 2), _gpu("w", w, torch.float32, 2), _gpu("state", state, x.dtype, 3), _contig("w", w), _contig("state", state)
+    T, width = x.shape
+    taps = w.shape[1]
+    if tuple(out.shape) != (T, width) or w.shape[0] != width or tuple(state.shape[1:]) != (taps - 1, width) or T != rows.rows or not 1 <= taps <= CONV_MAX_TAPS:
+        raise AlofaError("shape_mismatch", "convolution operands do not fit", f"out={tuple(out.shape)} x={tuple(x.shape)} w={tuple(w.shape)} state={tuple(state.shape)} rows={rows.rows}")
+    if bias is not None:
+        _gpu("bias", bias, torch.float32, 1), _contig("bias", bias)
+        if bias.shape[0] != width:
+            raise AlofaError("shape_mismatch", "one bias per channel", f"bias={tuple(bias.shape)}")
+    if out.data_ptr() == x.data_ptr():
+        raise AlofaError("invalid_argument", "the convolution does not run in place")
+    rows.fits("state", state)
+    _call("alofa_conv_bias_act", _ptr(out), _L(_rows("out", out)), _I(dtype_code(out)), _ptr(x), _L(_rows("x", x)), _I(dtype_code(x)), _ptr(w), _ptr(bias), _ptr(state),
+          _ptr(rows.slots), _ptr(rows.offsets), _ptr(rows.req_of_row), _I(T), _I(width), _I(taps), _I(int(silu)), _I(int(exact)), _stream())
+
+
+def conv_keep(state: torch.Tensor, x: torch.Tensor, rows: RowsOfRequests) -> None:
+    """``keep_last_rows`` for rows with a stride: state[slot] = the last inputs its request has seen once this step's rows are in."""
+    _gpu("state", state, x.dtype, 3), _gpu("x", x, None, 2), _contig("state", state)
+    if state.shape[2] != x.shape[1] or x.shape[0] != rows.rows or state.shape[1] > CONV_MAX_TAPS - 1:
+        raise AlofaError("shape_mismatch", "the kept rows do not fit", f"state={tuple(state.shape)} x={tuple(x.shape)} rows={rows.rows}")
+    rows.fits("state", state)
+    _call("alofa_conv_keep", _ptr(state), _ptr(x), _L(_rows("x", x)), _I(dtype_code(x)), _ptr(rows.slots), _ptr(rows.offsets), _I(rows.requests), _I(x.shape[1]),
+          _I(state.shape[1]), _stream())
+
+
+def ssd_operands(qf: torch.Tensor, kf: torch.Tensor, vf: torch.Tensor, decay: torch.Tensor, xbc: torch.Tensor, dt_raw: torch.Tensor, dt_bias: torch.Tensor,
+                 a_log: torch.Tensor, heads: int, groups: int, state: int, dv: int, exact: bool = False) -> None:
+    """What ``linear_recurrence`` takes for a state-space mixer, as float32 rows: with dt = softplus(dt_raw + dt_bias) per row and head, decay = exp(-exp(a_log) dt) for every
+    key channel of the head, kf = dt * B and qf = C of the head's group, vf = x. ``xbc`` [T, heads * dv + 2 * groups * state]: x, B, C side by side."""
+    T = xbc.shape[0]
+    for n, t, w in (("qf", qf, heads * state), ("kf", kf, heads * state), ("decay", decay, heads * state), ("vf", vf, heads * dv)):
+        _gpu(n, t, torch.float32, 2), _contig(n, t)
+        if tuple(t.shape) != (T, w):
+            raise AlofaError("shape_mismatch", "the float operands do not fit", f"operand={n} shape={tuple(t.shape)} rows={T} width={w}")
+    _gpu("xbc", xbc, None, 2), _gpu("dt_raw", dt_raw, xbc.dtype, 2), _gpu("dt_bias", dt_bias, torch.float32, 1), _gpu("a_log", a_log, torch.float32, 1)
+    _contig("dt_bias", dt_bias), _contig("a_log", a_log)
+    if xbc.shape[1] != heads * dv + 2 * groups * state or tuple(dt_raw.shape) != (T, heads) or dt_bias.shape[0] != heads or a_log.shape[0] != heads or heads % groups:
+        raise AlofaError("shape_mismatch", "the rows do not fit", f"xbc={tuple(xbc.shape)} dt={tuple(dt_raw.shape)} heads={heads} groups={groups} state={state} dv={dv}")
+    _call("alofa_ssd_operands", _ptr(qf), _ptr(kf), _ptr(vf), _ptr(decay), _ptr(xbc), _L(_rows("xbc", xbc)), _ptr(dt_raw), _L(_rows("dt_raw", dt_raw)), _I(dtype_code(xbc)),
+          _ptr(dt_bias), _ptr(a_log), _L(T), _I(heads), _I(groups), _I(state), _I(dv), _I(int(exact)), _stream())
+
+
+def ssd_finish(out: torch.Tensor, o: torch.Tensor, x: torch.Tensor, z: torch.Tensor, skip: torch.Tensor, weight: torch.Tensor, heads: int, dv: int, norm_parts: int,
+               eps: float, exact: bool = False, parts: int = 1) -> None:
+    """out = rms_parts((o + skip[head] * x) * silu(z)) * weight: the read-outs ``o`` float32 [T, heads * dv] (or [P, T, heads * dv], the first ``parts`` added), the
+    values ``x`` and gates ``z`` [T, heads * dv] rows (strides allowed), ``skip`` float32 [heads], the row normed in ``norm_parts`` equal parts, ``weight`` float32 [heads * dv]."""
+    _gpu("out", out, None, 2), _gpu("o", o, torch.float32), _contig("o", o), _gpu("x", x, out.dtype, 2), _gpu("z", z, out.dtype, 2)
+    _gpu("skip", skip, torch.float32, 1), _gpu("weight", weight, torch.float32, 1), _contig("skip", skip), _contig("weight", weight)
+    part_stride = 0
+    if o.dim() == 3:
+        if not 1 <= parts <= o.shape[0]:
+            raise AlofaError("shape_mismatch", "more parts than the read-outs have room for", f"o={tuple(o.shape)} parts={parts}")
+        part_stride, o = o.stride(0), o[0]
+    elif o.dim() != 2 or parts != 1:
+        raise AlofaError("shape_mismatch", "read-outs are [T, heads * dv] or parts of that", f"o={tuple(o.shape)} parts={parts}")
+    T, inner = o.shape[0], heads * dv
+    if o.shape[1] != inner or any(tuple(t.shape) != (T, inner) for t in (out, x, z)) or skip.shape[0] != heads or weight.shape[0] != inner or norm_parts <= 0 or inner % norm_parts:
+        raise AlofaError("shape_mismatch", "the rows do not fit", f"out={tuple(out.shape)} o={tuple(o.shape)} x={tuple(x.shape)} z={tuple(z.shape)} heads={heads} dv={dv} norm_parts={norm_parts}")
+    _call("alofa_ssd_finish", _ptr(out), _L(_rows("out", out)), _ptr(o), _I(parts), _L(part_stride), _ptr(x), _L(_rows("x", x)), _ptr(z), _L(_rows("z", z)), _I(dtype_code(out)),
+          _ptr(skip), _ptr(weight), _L(T), _I(heads), _I(dv), _I(norm_parts), _F(eps), _I(int(exact)), _stream())
+
+
+def rms_pair_sum(out: torch.Tensor, a: torch.Tensor, wa: torch.Tensor, sa: float, b: torch.Tensor, wb: torch.Tensor, sb: float, eps: float, exact: bool = False) -> None:
+    """out[t] = sa * a[t] / rms(a[t]) * wa + sb * b[t] / rms(b[t]) * wb, all float32 [T, h] (weights [h]); rms(x) = sqrt(mean(x^2) + eps). ``out`` may be ``a`` or ``b``."""
+    for n, t in (("out", out), ("a", a), ("b", b)):
+        _gpu(n, t, torch.float32, 2), _contig(n, t)
+    _gpu("wa", wa, torch.float32, 1), _gpu("wb", wb, torch.float32, 1), _contig("wa", wa), _contig("wb", wb)
+    T, h = out.shape
+    if a.shape != out.shape or b.shape != out.shape or wa.shape[0] != h or wb.shape[0] != h:
+        raise AlofaError("shape_mismatch", "two branches of the output's shape, one weight per channel each", f"out={tuple(out.shape)} a={tuple(a.shape)} b={tuple(b.shape)}")
+    _call("alofa_rms_pair_sum", _ptr(out), _ptr(a), _ptr(wa), _F(sa), _ptr(b), _ptr(wb), _F(sb), _L(T), _I(h), _F(eps), _I(int(exact)), _stream())

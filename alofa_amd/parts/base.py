@@ -81,15 +81,19 @@ class CacheTensor:
     standing for the tokens of the page: (kv_heads, SLOT, head_dim) lays the tokens of a page out
     one after the other per head; (kv_heads, head_dim, SLOT) keeps them transposed; (SLOT, width)
     is one vector per token. The cache manager allocates [pages, *dims] with the page size in
-    SLOT's place. ``dtype`` None: the runtime's activation dtype."""
+    SLOT's place. ``dtype`` None: the runtime's activation dtype. ``every`` n > 1: the tensor keeps one entry per run of n
+    tokens instead of one per token (a summary of the run); the run that begins at token t of a page has place t // n there,
+    so a page has (page size - 1) // n + 1 places in SLOT's place."""
     name: str
     dims: tuple
     dtype: Optional[torch.dtype] = None
+    every: int = 1
 
     def page_shape(self, block_size: int) -> tuple:
-        if tuple(self.dims).count(SLOT) != 1 or any(d <= 0 for d in self.dims if d != SLOT):
-            raise AlofaError("invalid_argument", "a cache tensor's dims hold positive sizes and SLOT exactly once", f"name={self.name} dims={self.dims}")
-        return tuple(block_size if d == SLOT else int(d) for d in self.dims)
+        if tuple(self.dims).count(SLOT) != 1 or any(d <= 0 for d in self.dims if d != SLOT) or self.every < 1:
+            raise AlofaError("invalid_argument", "a cache tensor's dims hold positive sizes and SLOT exactly once", f"name={self.name} dims={self.dims} every={self.every}")
+        places = block_size if self.every == 1 else (block_size - 1) // self.every + 1
+        return tuple(places if d == SLOT else int(d) for d in self.dims)
 
 
 @dataclass(frozen=True)

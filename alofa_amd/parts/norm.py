@@ -11,17 +11,19 @@ from .base import Norm, register_part
 
 
 class RMSNorm(Norm):
-    """params: name (tensor name), width, eps."""
+    """params: name (tensor name), width, eps; scalar (True: the weight is one number for all channels, a tensor without
+    dimensions; it is spread over the width when the weights are loaded, so every kernel that takes an RMSNorm takes this one)."""
 
     @classmethod
     def tensors(cls, spec):
-        return {spec.params["name"]: TensorRule((spec.params["width"],), "norm")}
+        return {spec.params["name"]: TensorRule(() if spec.params.get("scalar", False) else (spec.params["width"],), "norm")}
 
     def __init__(self, spec, weights, rt):
         super().__init__(spec, weights, rt)
         self.eps = float(spec.params["eps"])
         self.width = int(spec.params["width"])
-        self.weight = rt.vector(weights[spec.params["name"]])
+        weight = weights[spec.params["name"]]
+        self.weight = rt.vector(weight.float().reshape(1).repeat(self.width) if spec.params.get("scalar", False) else weight)
 
     def as_rmsnorm(self):
         return self.weight, self.eps

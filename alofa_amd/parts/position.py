@@ -18,9 +18,14 @@ from .base import PositionEncoding, register_part
 
 
 class Rotary(PositionEncoding):
-    """params: theta, head_dim, pairing ("half"), dims (how many of a head's first channels are rotated, default all
-    of them: channel i < dims/2 is paired with i + dims/2, the angle is p * theta^(-2i/dims), the channels from
-    ``dims`` on pass unchanged), factor (every frequency is divided by it: positions stretched linearly; default 1).
+    """params: theta, head_dim, pairing ("half": channel i < dims/2 is paired with i + dims/2; "neighbours": channel 2i with
+    2i + 1), dims (how many of a head's first channels are rotated, default all of them; the angle of pair i is
+    p * theta^(-2i/dims), the channels from ``dims`` on pass unchanged), factor (every frequency is divided by it: positions
+    stretched linearly; default 1), stretch ({factor, original, fast, slow}: frequencies stretched by wavelength: with
+    dim(t) = dims ln(original / (2 pi t)) / (2 ln theta), lo = max(floor(dim(fast)), 0), hi = min(ceil(dim(slow)), dims - 1) and
+    ramp_i = clamp((i - lo) / max(hi - lo, 0.001), 0, 1), pair i turns at f_i / factor * ramp_i + f_i (1 - ramp_i), and cos and sin
+    are multiplied by 0.1 ln(factor) + 1), frequencies ("reciprocal": 1 / float32(theta^(2i/dims)) in float32, the default;
+    "direct": theta^(-2i/dims) formed in float64 and rounded once).
 
     The kernels pair channel j with j + head_dim/2. With dims < head_dim the table holds the angle zero for the pairs
     beyond dims/2, and ``channel_order`` names the order of a head's channels in which the design's pairs lie that
@@ -37,8 +42,16 @@ class Rotary(PositionEncoding):
             raise AlofaError("invalid_argument", "the factor that stretches positions is positive", f"factor={self.factor}")
         if self.dims <= 0 or self.dims % 2 or self.dims > self.head_dim:
             raise AlofaError("unsupported", "rotated channels: an even count, at most the head's size", f"dims={self.dims} head_dim={self.head_dim}")
-        if spec.params.get("pairing", "half") != "half":
-            raise AlofaError("unsupported", "only the half-split pairing (j, j + d/2) is built", f"pairing={spec.params['pairing']}")
+        self.pairing = spec.params.get("pairing", "half")
+        if self.pairing not in ("half", "neighbours"):
+            raise AlofaError("unsupported", "pairs are (j, j + dims/2) or (2j, 2j + 1)", f"pairing={spec.params['pairing']}")
+        self.direct = spec.params.get("frequencies", "reciprocal") == "direct"
+        self.stretch = spec.params.get("stretch")
+        if self.stretch is not None:
+            st = {k: float(self.stretch[k]) for k in ("factor", "original", "fast", "slow")}
+            if not (st["factor"] > 0 and st["original"] > 0 and st["fast"] > 0 and st["slow"] > 0 and self.theta > 1):
+                raise AlofaError("invalid_argument", "a stretch by wavelength takes positive numbers and a base above one", f"stretch={self.stretch} theta={self.theta}")
+            self.stretch = st
         if self.head_dim <= 0 or self.head_dim % 2:
             raise AlofaError("unsupported", "head dimension must be positive and even", f"head_dim={self.head_dim}")
 
@@ -46,17 +59,36 @@ class Rotary(PositionEncoding):
         half = self.head_dim // 2
         inv = np.zeros(half, dtype=np.float32)      # (pairs beyond dims/2 keep the angle zero: they pass unchanged)
         for i in range(self.dims // 2):
+            if self.direct:
+                inv[i] = np.float32(self._frequency(i))
+                continue
             inv[i] = np.float32(1.0) / np.float32(math.pow(self.theta, (2.0 * i) / self.dims))
             if self.factor != 1.0:
                 inv[i] = inv[i] / np.float32(self.factor)
         ang = np.arange(n_positions, dtype=np.float32)[:, None] * inv[None, :]
         ang = ang.astype(np.float32).astype(np.float64)
-        return np.cos(ang).astype(np.float32), np.sin(ang).astype(np.float32)
+        mag = 1.0 if self.stretch is None else 0.1 * math.log(self.stretch["factor"]) + 1.0
+        return (np.cos(ang) * mag).astype(np.float32), (np.sin(ang) * mag).astype(np.float32)
+
+    def _frequency(self, i: int) -> float:
+        """Pair i's frequency in float64, with the linear factor and the stretch by wavelength."""
+        f = math.pow(self.theta, -2.0 * i / self.dims) / self.factor
+        st = self.stretch
+        if st is not None:
+            def dim_of(turns):
+                return self.dims * math.log(st["original"] / (2.0 * math.pi * turns)) / (2.0 * math.log(self.theta))
+            lo = max(math.floor(dim_of(st["fast"])), 0)
+            hi = min(math.ceil(dim_of(st["slow"])), self.dims - 1)
+            ramp = min(max((i - lo) / max(hi - lo, 0.001), 0.0), 1.0)
+            f = f / st["factor"] * ramp + f * (1.0 - ramp)
+        return f
 
     def channel_order(self):
-        if self.dims == self.head_dim:
+        if self.dims == self.head_dim and self.pairing == "half":
             return None
         r, rest = self.dims // 2, (self.head_dim - self.dims) // 2
+        if self.pairing == "neighbours":
+            return [*range(0, self.dims, 2), *range(self.dims, self.dims + rest), *range(1, self.dims, 2), *range(self.dims + rest, self.head_dim)]
         return [*range(r), *range(self.dims, self.dims + rest), *range(r, self.dims), *range(self.dims + rest, self.head_dim)]
 
     @classmethod
@@ -70,7 +102,7 @@ class Rotary(PositionEncoding):
         """One table per (theta, head size) serves every layer of the model (kept on the runtime).
         A table that has to grow is replaced; the old one is kept alive, since a captured graph
         may still read it (for positions it covers)."""
-        key = ("rotary", self.theta, self.head_dim, self.dims, self.factor)
+        key = ("rotary", self.theta, self.head_dim, self.dims, self.factor, self.direct, tuple(sorted(self.stretch.items())) if self.stretch else None)
         have = self.rt.shared.get(key)
         if have is None or have[0].shape[0] < n_positions:
             n = max(n_positions, 2 * have[0].shape[0] if have else 0)

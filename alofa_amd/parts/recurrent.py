@@ -18,6 +18,11 @@ matrix_memory   exponential gates per head kept in range by a running maximum m 
                 normaliser n_t likewise with k alone; o = S_t^T q / (max(|n_t . q|, exp(-m_t)) + 1e-6), q scaled by dk^(-1/2); o / rms(o)
                 per head, times a weight per channel, times sigmoid(gate), output projection.
 
+state_space     a decay per head and step made of a step size (the "state-space duality" form): one projection gives z, x, B, C and dt side by side;
+                x, B, C pass a short causal convolution with bias and silu; dt = softplus(dt + bias); S_t = exp(-exp(A_log) dt_t) S_(t-1) + dt_t B_t x_t^T
+                (S [state, value_dim] per head; B and C shared by the heads of a group), y_t = S_t^T C_t + D x_t; y times silu(z), an RMS norm over
+                each of several equal parts of the row, a weight, output projection. The convolution's last inputs are a second piece of state.
+
 Projections and gates run in the activation dtype; decays, the state, the read-out and the head norms in float32.
 Every one of them takes ``out=`` (see ``Mixer.forward``)."""
 from __future__ import annotations
@@ -264,6 +269,82 @@ class MatrixMemory(RecurrentMixer):
             ops.gemm(residual, y, self.w_o, add_to_out=True, exact=exact)
 
 
+class ConvTail(Mixer):
+    """The last taps - 1 inputs of a short convolution inside a mixer: a second piece of state per request beside the mixer's own."""
+    capturable = True
+
+    def __init__(self, keep: int, width: int, dtype, rt):
+        self.keep, self.width, self.dtype, self.rt, self.spec = keep, width, dtype, rt, None
+
+    def state_need(self):
+        return StateNeed((self.keep, self.width), self.dtype) if self.keep > 0 else None
+
+
+class StateSpace(RecurrentMixer):
+    """params: prefix, hidden, heads, value_dim (a head's channels), state (N), groups, taps, norm_parts, eps. Tensors: prefix + in
+    [2 * heads * value_dim + 2 * groups * state + heads, hidden], conv [heads * value_dim + 2 * groups * state, taps], conv.b, dt_bias, A_log, D [heads],
+    norm [heads * value_dim], o."""
+
+    @classmethod
+    def tensors(cls, spec):
+        p = spec.params
+        pre, h, H, dv, N, G = p["prefix"], p["hidden"], p["heads"], p["value_dim"], p["state"], p["groups"]
+        inner, conv = H * dv, H * dv + 2 * G * N
+        return {pre + "in": TensorRule((2 * inner + 2 * G * N + H, h), "fan_in"), pre + "conv": TensorRule((conv, p["taps"]), "filter"),
+                pre + "conv.b": TensorRule((conv,), "bias"), pre + "dt_bias": TensorRule((H,), "bias"), pre + "A_log": TensorRule((H,), "log_rate"),
+                pre + "D": TensorRule((H,), "norm"), pre + "norm": TensorRule((inner,), "norm"), pre + "o": TensorRule((h, inner), "fan_in")}
+
+    def __init__(self, spec, weights, rt):
+        p = spec.params
+        super().__init__(PartSpec(spec.kind, {**p, "key_dim": p["state"]}), weights, rt)
+        self.spec = spec
+        pre = p["prefix"]
+        self.groups, self.taps, self.norm_parts = int(p["groups"]), int(p["taps"]), int(p["norm_parts"])
+        self.inner = self.heads * self.dv
+        self.conv_width = self.inner + 2 * self.groups * self.dk
+        if self.groups <= 0 or self.heads % self.groups or self.norm_parts <= 0 or self.inner % self.norm_parts or not 1 <= self.taps <= ops.CONV_MAX_TAPS:
+            raise AlofaError("invalid_argument", "groups divide the heads, the norm's parts divide the row, and the convolution has 1 to 16 taps",
+                             f"heads={self.heads} groups={self.groups} norm_parts={self.norm_parts} taps={self.taps}")
+        w_in = weights[pre + "in"]
+        if w_in.shape[0] % 8:      # (rows of the projection stay 16-byte aligned)
+            w_in = torch.cat([w_in, torch.zeros((8 - w_in.shape[0] % 8, w_in.shape[1]), dtype=w_in.dtype)])
+        self.w_in, self.w_o = rt.matrix(w_in), rt.matrix(weights[pre + "o"])
+        self.conv_w, self.conv_b = rt.vector(weights[pre + "conv"]), rt.vector(weights[pre + "conv.b"])
+        self.dt_bias, self.a_log, self.skip = rt.vector(weights[pre + "dt_bias"]), rt.vector(weights[pre + "A_log"]), rt.vector(weights[pre + "D"])
+        self.norm = rt.vector(weights[pre + "norm"])
+        self.tail = ConvTail(self.taps - 1, self.conv_width, rt.dtype, rt)
+
+    def stateful_parts(self):
+        return [self, self.tail]
+
+    def forward(self, ctx, where, x, residual, out=None):
+        T, H, N, dv, inner = x.shape[0], self.heads, self.dk, self.dv, self.inner
+        entry, k = where if isinstance(where, tuple) else (where, 0)
+        exact, rows = self.rt.exact, rows_of_requests(ctx)
+        proj = ctx.scratch("recurrent_proj", (T, self.w_in.shape[0]), self.rt.dtype)
+        ops.gemm(proj, x, self.w_in, exact=exact)
+        z, raw, dt = proj[:, :inner], proj[:, inner:inner + self.conv_width], proj[:, inner + self.conv_width:inner + self.conv_width + H]
+        xbc = ctx.scratch("state_space_conv", (T, self.conv_width), self.rt.dtype)
+        if self.taps > 1:
+            tail = ctx.state((entry, k + 1))
+            ops.conv_bias_act(xbc, raw, self.conv_w, self.conv_b, tail, rows, silu=True, exact=exact)
+            ops.conv_keep(tail, raw, rows)
+        else:
+            none = ctx.scratch("conv_no_state", (ctx.fn.cache.max_requests, 0, self.conv_width), self.rt.dtype)
+            ops.conv_bias_act(xbc, raw, self.conv_w, self.conv_b, none, rows, silu=True, exact=exact)
+        qf, kf = ctx.scratch("memory_q", (T, H * N), torch.float32), ctx.scratch("memory_k", (T, H * N), torch.float32)
+        vf, decay = ctx.scratch("memory_v", (T, inner), torch.float32), ctx.scratch("recurrent_decay", (T, H * N), torch.float32)
+        ops.ssd_operands(qf, kf, vf, decay, xbc, dt, self.dt_bias, self.a_log, H, self.groups, N, dv, exact)
+        o = self._readouts(ctx, T)
+        parts = ops.linear_recurrence(o, qf, kf, vf, ctx.state((entry, k)), rows, H, N, dv, ops.DECAY_GIVEN, decay)
+        y = ctx.scratch("recurrent_gated", (T, inner), self.rt.dtype)
+        ops.ssd_finish(y, o, xbc[:, :inner], z, self.skip, self.norm, H, dv, self.norm_parts, self.eps, exact, parts=parts)
+        if out is not None:
+            ops.gemm(out, y, self.w_o, exact=exact)
+        else:
+            ops.gemm(residual, y, self.w_o, add_to_out=True, exact=exact)
+
+
 MIXES = ("r", "k", "v", "g", "w")
 
 
@@ -348,7 +429,9 @@ class TimeMix(RecurrentMixer):
 
 class ParallelMixers(Mixer):
     """Several mixers side by side that read the same rows; the result is the sum of theirs, each times its scale.
-    params: branches (PartSpecs of mixers that take ``out=``), scales (one per branch), hidden."""
+    params: branches (PartSpecs of mixers that take ``out=``), scales (one per branch), hidden; norms (optional: one tensor name per
+    branch, a weight [hidden] each: every branch's result passes an RMS norm over the width with that weight before the sum; two
+    branches) and eps."""
 
     @classmethod
     def tensors(cls, spec):
@@ -356,6 +439,8 @@ class ParallelMixers(Mixer):
         out = {}
         for b in spec.params["branches"]:
             out.update(tensors_of("mixer", b))
+        for name in spec.params.get("norms") or ():
+            out[name] = TensorRule((spec.params["hidden"],), "norm")
         return out
 
     def __init__(self, spec, weights, rt):
@@ -366,6 +451,10 @@ class ParallelMixers(Mixer):
         self.scales = [float(s) for s in p["scales"]]
         if not self.branches or len(self.scales) != len(self.branches):
             raise AlofaError("invalid_argument", "one scale per branch, and at least one branch", f"branches={len(self.branches)} scales={len(self.scales)}")
+        self.norms = [rt.vector(weights[n]) for n in p.get("norms") or ()]
+        self.eps = float(p.get("eps", 1e-6))
+        if self.norms and (len(self.norms) != 2 or len(self.branches) != 2):
+            raise AlofaError("unsupported", "branches that are normed before the sum come in pairs, a norm each", f"branches={len(self.branches)} norms={len(self.norms)}")
 
     @property
     def capturable(self):
@@ -386,6 +475,13 @@ class ParallelMixers(Mixer):
             b.forward(ctx, (entry, k), x, residual, out=buf)
             k += len(b.stateful_parts())
             outs.append(buf)
+        if self.norms:
+            if out is not None:
+                ops.rms_pair_sum(out, outs[0], self.norms[0], self.scales[0], outs[1], self.norms[1], self.scales[1], self.eps, self.rt.exact)
+            else:
+                ops.rms_pair_sum(outs[0], outs[0], self.norms[0], self.scales[0], outs[1], self.norms[1], self.scales[1], self.eps, self.rt.exact)
+                ops.add_scaled(residual, outs[0], 1.0, exact=self.rt.exact)
+            return
         target = residual
         if out is not None:
             out.zero_()
@@ -400,5 +496,6 @@ register_part("mixer", "gated_linear", GatedLinearAttention)
 register_part("mixer", "time_mix", TimeMix)
 register_part("mixer", "lightning_attention", LightningAttention)
 register_part("mixer", "matrix_memory", MatrixMemory)
+register_part("mixer", "state_space", StateSpace)
 register_part("mixer", "parallel", ParallelMixers)
 register_part("conv", "token_shift", TokenShift)
