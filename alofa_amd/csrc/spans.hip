@@ -277,6 +277,218 @@ __global__ void __launch_bounds__(256) span_attention_kernel(T* __restrict__ out
   }
 }
 
+// ---- the matrix-core kernel: a wavefront per (16 rows of one request, head), bfloat16 ---------------------------
+// Both products are taken transposed (v_mfma_f32_16x16x32_bf16; lane l: A row and B column l % 16, reduction slots 8 (l / 16) .. + 7,
+// D column l % 16 and rows 4 (l / 16) .. + 3), so a lane stays with one query row throughout:
+//   S^T[key, q] = K[key, :] . Q[q, :]       A = keys straight from the pages (16 bytes a lane), B = queries (registers)
+//   O^T[c, q] += V^T[c, key] * P^T[key, q]   A = transposed values straight from the pages (two runs of four keys a lane), B = weights
+// Keys are walked in tiles of 32 that start at multiples of 32: after the first product lane l holds, for query l % 16, the scores of
+// keys 4 g + r and 16 + 4 g + r (g = l / 16, r = 0..3), which are the eight reduction slots of the second product when the values are read
+// in that order, so the weights never leave their registers. The four lanes of a query meet for the tile's maximum; the running
+// maximum, the weights' sum and the scores are float. Then the blocks behind the window, 32 at a time, the same way (their places
+// are looked up one by one). The sink joins the denominator at the end; the gate rides on the store.
+typedef __bf16 span_bf16x8 __attribute__((ext_vector_type(8)));
+typedef float span_f32x4 __attribute__((ext_vector_type(4)));
+
+struct SpanFastArgs {
+  int64_t out_stride, q_stride, gate_stride;
+  const int32_t* tiles;        // [n_tiles, 3]: request, first row, rows (<= 16); nullptr: tile t is row t alone, of request req_of_token[t] (or t)
+  const int32_t* table;
+  int max_blocks;
+  const int32_t* pool_table;
+  int pool_max_blocks;
+  const int32_t* req_of_token;
+  const int32_t* positions;
+  int n_tiles, heads, kv_heads, bs_shift, window, P, places, dv_true;
+  float scale;
+  const float* bias;
+  int bias_len;
+  const float* sink;
+  int gate_kind;
+};
+
+template <int DT>
+__global__ void __launch_bounds__(256) span_attention_mfma_kernel(bf16_t* __restrict__ out, const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_cache,
+                                                                  const bf16_t* __restrict__ v_cache, const bf16_t* __restrict__ pk, const bf16_t* __restrict__ pv,
+                                                                  const bf16_t* __restrict__ gate, SpanFastArgs a) {
+  constexpr int d = DT * 16, DS = (d + 31) / 32;
+  constexpr float kLow = -1e30f;
+  const int lane = threadIdx.x % kWave, col = lane % 16, grp = lane / 16;
+  const int h = blockIdx.y * 4 + threadIdx.x / kWave;
+  if (h >= a.heads) return;
+  const int g = h / (a.heads / a.kv_heads), S = 1 << a.bs_shift;
+  int r, row0, n;
+  if (a.tiles) {
+    r = a.tiles[3 * blockIdx.x], row0 = a.tiles[3 * blockIdx.x + 1], n = a.tiles[3 * blockIdx.x + 2];
+  } else {
+    row0 = blockIdx.x, n = 1, r = a.req_of_token ? a.req_of_token[row0] : row0;
+  }
+  const bool valid = col < n;
+  const int row = row0 + (valid ? col : 0);
+  const int p = a.positions[row];
+  const int p_first = a.positions[row0], p_last = a.positions[row0 + n - 1];
+  const int W = a.window;
+  const int lo = (W > 0 && p_first - W + 1 > 0) ? p_first - W + 1 : 0;
+  const int32_t* tab = a.table + static_cast<int64_t>(r) * a.max_blocks;
+
+  span_bf16x8 qf[DS];
+#pragma unroll
+  for (int s = 0; s < DS; ++s) {
+    const int c = s * 32 + grp * 8;
+    qf[s] = span_bf16x8{};
+    if (valid && c < d) qf[s] = *reinterpret_cast<const span_bf16x8*>(q + static_cast<int64_t>(row) * a.q_stride + static_cast<int64_t>(h) * d + c);
+  }
+  span_f32x4 acc[DT];
+#pragma unroll
+  for (int o = 0; o < DT; ++o) acc[o] = span_f32x4{0.f, 0.f, 0.f, 0.f};
+  float m = kLow, l = 0.f;
+  const float* bias = a.bias ? a.bias + static_cast<int64_t>(h) * a.bias_len : nullptr;
+
+  // one tile of 32 entries: scores sc[u][r] for entries e(u, r) = t0 + 16 u + 4 grp + r of query col, their visibility, and the second product
+  auto softmax_step = [&](span_f32x4 (&sc)[2], const bool (&seen)[2][4], auto&& values) {
+    float top = kLow;
+#pragma unroll
+    for (int u = 0; u < 2; ++u)
+#pragma unroll
+      for (int x = 0; x < 4; ++x) top = fmaxf(top, seen[u][x] ? sc[u][x] : kLow);
+    top = rows_max(top);
+    const float m_new = fmaxf(m, top), alpha = __expf(m - m_new);
+    span_bf16x8 w;
+    float sum = 0.f;
+#pragma unroll
+    for (int u = 0; u < 2; ++u)
+#pragma unroll
+      for (int x = 0; x < 4; ++x) {
+        const float e = seen[u][x] ? __expf(sc[u][x] - m_new) : 0.f;
+        sum += e;
+        w[4 * u + x] = static_cast<__bf16>(e);
+      }
+    l = l * alpha + sum;
+    m = m_new;
+#pragma unroll
+    for (int o = 0; o < DT; ++o) {
+      acc[o] *= alpha;
+      acc[o] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(values(o), w, acc[o], 0, 0, 0);
+    }
+  };
+
+  // ---- the window's tokens
+  for (int t0 = (lo / 32) * 32; t0 <= p_last; t0 += 32) {
+    span_f32x4 sc[2];
+    bool seen[2][4];
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      int key = t0 + 16 * u + col;      // (the key this lane fetches for the first product: clamped to one whose page is held)
+      key = key < lo ? lo : (key > p_last ? p_last : key);
+      const bf16_t* krow = k_cache + ((static_cast<int64_t>(tab[key >> a.bs_shift]) * a.kv_heads + g) * S + (key & (S - 1))) * d;
+      sc[u] = span_f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int s = 0; s < DS; ++s) {
+        const int c = s * 32 + grp * 8;
+        span_bf16x8 kf = span_bf16x8{};
+        if (c < d) kf = *reinterpret_cast<const span_bf16x8*>(krow + c);
+        sc[u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[s], sc[u], 0, 0, 0);
+      }
+#pragma unroll
+      for (int x = 0; x < 4; ++x) {
+        const int j = t0 + 16 * u + 4 * grp + x, dist = p - j;
+        seen[u][x] = valid && dist >= 0 && (W <= 0 || dist < W);
+        float b = 0.f;
+        if (bias && seen[u][x]) b = bias[dist < a.bias_len ? dist : a.bias_len - 1];
+        sc[u][x] = sc[u][x] * a.scale + b;
+      }
+    }
+    softmax_step(sc, seen, [&](int o) {
+      span_bf16x8 vf;
+#pragma unroll
+      for (int u = 0; u < 2; ++u) {
+        int j = t0 + 16 * u + 4 * grp;      // (four keys of one page; clamped to a run whose page is held)
+        j = j < (lo & ~3) ? (lo & ~3) : (j > (p_last & ~3) ? (p_last & ~3) : j);
+        const bf16_t* vrow = v_cache + ((static_cast<int64_t>(tab[j >> a.bs_shift]) * a.kv_heads + g) * d + o * 16 + col) * S + (j & (S - 1));
+        const uint2 four = *reinterpret_cast<const uint2*>(vrow);
+        const uint32_t two[2] = {four.x, four.y};
+#pragma unroll
+        for (int x = 0; x < 4; ++x) vf[4 * u + x] = __builtin_bit_cast(__bf16, static_cast<uint16_t>(two[x / 2] >> (16 * (x % 2))));
+      }
+      return vf;
+    });
+  }
+
+  // ---- the blocks wholly behind the window
+  const int n_blk_tile = (a.pool_table && W > 0 && p_last - W + 1 >= a.P) ? (p_last - W + 1) / a.P : 0;
+  if (n_blk_tile > 0) {
+    const int32_t* ptab = a.pool_table + static_cast<int64_t>(r) * a.pool_max_blocks;
+    const int mine = (p - W + 1 >= a.P) ? (p - W + 1) / a.P : 0;      // how many blocks this lane's query sees
+    auto place_of = [&](int e, int64_t& page, int& place) {
+      e = e < n_blk_tile ? e : n_blk_tile - 1;
+      const int first = e * a.P;
+      page = ptab[first >> a.bs_shift];
+      place = (first & (S - 1)) / a.P;
+    };
+    for (int e0 = 0; e0 < n_blk_tile; e0 += 32) {
+      span_f32x4 sc[2];
+      bool seen[2][4];
+#pragma unroll
+      for (int u = 0; u < 2; ++u) {
+        int64_t page;
+        int place;
+        place_of(e0 + 16 * u + col, page, place);
+        const bf16_t* krow = pk + ((page * a.kv_heads + g) * a.places + place) * d;
+        sc[u] = span_f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int s = 0; s < DS; ++s) {
+          const int c = s * 32 + grp * 8;
+          span_bf16x8 kf = span_bf16x8{};
+          if (c < d) kf = *reinterpret_cast<const span_bf16x8*>(krow + c);
+          sc[u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[s], sc[u], 0, 0, 0);
+        }
+#pragma unroll
+        for (int x = 0; x < 4; ++x) {
+          seen[u][x] = valid && e0 + 16 * u + 4 * grp + x < mine;
+          sc[u][x] *= a.scale;
+        }
+      }
+      int64_t pages[8];
+      int places[8];
+#pragma unroll
+      for (int u = 0; u < 2; ++u)
+#pragma unroll
+        for (int x = 0; x < 4; ++x) place_of(e0 + 16 * u + 4 * grp + x, pages[4 * u + x], places[4 * u + x]);
+      softmax_step(sc, seen, [&](int o) {
+        span_bf16x8 vf;
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+          vf[i] = __builtin_bit_cast(__bf16, pv[((pages[i] * a.kv_heads + g) * d + o * 16 + col) * a.places + places[i]]);
+        return vf;
+      });
+    }
+  }
+
+  float total = rows_sum(l);
+  if (a.sink) {
+    const float sk = a.sink[h], m_f = fmaxf(m, sk), alpha = __expf(m - m_f);
+    total = total * alpha + __expf(sk - m_f);
+#pragma unroll
+    for (int o = 0; o < DT; ++o) acc[o] *= alpha;
+  }
+  if (!valid) return;
+  const float inv = 1.f / total;
+  bf16_t* orow = out + static_cast<int64_t>(row) * a.out_stride + static_cast<int64_t>(h) * d;
+  const bf16_t* grow = a.gate_kind ? gate + static_cast<int64_t>(row) * a.gate_stride : nullptr;
+  const float head_gate = a.gate_kind == 2 ? 1.f / (1.f + __expf(-bf16_to_f32(grow[h]))) : 1.f;
+#pragma unroll
+  for (int o = 0; o < DT; ++o) {
+    float y[4];
+#pragma unroll
+    for (int x = 0; x < 4; ++x) {
+      const int c = o * 16 + 4 * grp + x;
+      y[x] = acc[o][x] * inv * head_gate;
+      if (a.gate_kind == 1) y[x] = c < a.dv_true ? y[x] / (1.f + __expf(-bf16_to_f32(grow[static_cast<int64_t>(h) * a.dv_true + c]))) : 0.f;
+    }
+    *reinterpret_cast<uint2*>(orow + o * 16 + 4 * grp) = uint2{pack_bf16x2(y[0], y[1]), pack_bf16x2(y[2], y[3])};
+  }
+}
+
 // out[t, h, :] *= sigmoid(gate[t, h]) (one gate per head) or sigmoid(gate[t, h, :]) (one per channel): what the matrix-core
 // attention kernels leave, on its way to the output projection.
 template <typename T>
@@ -363,6 +575,42 @@ extern "C" int alofa_span_attention(void* out, int64_t out_stride, const void* q
   else ALOFA_SPAN(bf16_t, float);
 #undef ALOFA_SPAN
   return check_launch("span_attention");
+}
+
+template <int DT>
+static void launch_span_mfma(dim3 grid, hipStream_t stream, void* out, const void* q, const void* k_cache, const void* v_cache, const void* pk, const void* pv, const void* gate,
+                             const SpanFastArgs& a) {
+  span_attention_mfma_kernel<DT><<<grid, 256, 0, stream>>>(static_cast<bf16_t*>(out), static_cast<const bf16_t*>(q), static_cast<const bf16_t*>(k_cache), static_cast<const bf16_t*>(v_cache),
+                                                           static_cast<const bf16_t*>(pk), static_cast<const bf16_t*>(pv), static_cast<const bf16_t*>(gate), a);
+}
+
+// bfloat16 on the matrix cores: heads of d = dv channels in steps of 16, pages of a power of two of at least 8 tokens, rows 16-byte aligned.
+extern "C" int alofa_span_attention_mfma(void* out, int64_t out_stride, const void* q, int64_t q_stride, const void* k_cache, const void* v_cache, const void* pk, const void* pv,
+                                         const int32_t* tiles, int n_tiles, const int32_t* table, int max_blocks, const int32_t* pool_table, int pool_max_blocks,
+                                         const int32_t* req_of_token, const int32_t* positions, int heads, int kv_heads, int d, int dv_true, int block_size, int window, int P,
+                                         int places, float scale, const float* bias, int bias_len, const float* sink, const void* gate, int64_t gate_stride, int gate_kind,
+                                         hipStream_t stream) {
+  ALOFA_REQUIRE(n_tiles >= 0 && heads > 0 && kv_heads > 0 && heads % kv_heads == 0, "span_attention_mfma: tiles=%d heads=%d kv_heads=%d (kv_heads must divide heads)", n_tiles, heads, kv_heads);
+  ALOFA_REQUIRE(d >= 16 && d <= 256 && d % 16 == 0 && dv_true > 0 && dv_true <= d, "span_attention_mfma: head size %d (16 to 256 in steps of 16), of which %d value channels count", d, dv_true);
+  ALOFA_REQUIRE(block_size >= 8 && (block_size & (block_size - 1)) == 0 && max_blocks > 0 && window >= 0, "span_attention_mfma: pages of a power of two of at least 8 tokens (block_size=%d), window=%d", block_size, window);
+  ALOFA_REQUIRE(pool_table == nullptr || (pk && pv && window > 0 && P > 0 && places == (block_size - 1) / P + 1 && pool_max_blocks > 0), "span_attention_mfma: pooled blocks need their pages, a window and P (P=%d places=%d)", P, places);
+  ALOFA_REQUIRE(bias == nullptr || bias_len > 0, "span_attention_mfma: an empty bias table");
+  ALOFA_REQUIRE(gate_kind >= 0 && gate_kind <= 2 && (gate_kind == 0 || gate != nullptr), "span_attention_mfma: no such gate (%d)", gate_kind);
+  ALOFA_REQUIRE(q_stride % 8 == 0 && out_stride % 4 == 0 && reinterpret_cast<uintptr_t>(q) % 16 == 0 && reinterpret_cast<uintptr_t>(out) % 8 == 0, "span_attention_mfma: rows must be 16-byte aligned");
+  if (n_tiles == 0) return 0;
+  int shift = 0;
+  while ((1 << shift) < block_size) ++shift;
+  SpanFastArgs a{out_stride, q_stride, gate_stride, tiles, table, max_blocks, pool_table, pool_max_blocks, req_of_token, positions, n_tiles, heads, kv_heads, shift, window,
+                 P, places, dv_true, scale, bias, bias_len, sink, gate_kind};
+  const dim3 grid(n_tiles, (heads + 3) / 4);
+  switch (d / 16) {
+#define ALOFA_SPAN_DT(N) case N: launch_span_mfma<N>(grid, stream, out, q, k_cache, v_cache, pk, pv, gate, a); break;
+    ALOFA_SPAN_DT(1) ALOFA_SPAN_DT(2) ALOFA_SPAN_DT(3) ALOFA_SPAN_DT(4) ALOFA_SPAN_DT(5) ALOFA_SPAN_DT(6) ALOFA_SPAN_DT(7) ALOFA_SPAN_DT(8)
+    ALOFA_SPAN_DT(9) ALOFA_SPAN_DT(10) ALOFA_SPAN_DT(11) ALOFA_SPAN_DT(12) ALOFA_SPAN_DT(13) ALOFA_SPAN_DT(14) ALOFA_SPAN_DT(15) ALOFA_SPAN_DT(16)
+#undef ALOFA_SPAN_DT
+    default: ALOFA_REQUIRE(false, "span_attention_mfma: head size %d", d);
+  }
+  return check_launch("span_attention_mfma");
 }
 
 extern "C" int alofa_head_gate(void* x, int64_t x_stride, const void* gate, int64_t gate_stride, int dtype, int64_t rows, int heads, int dv, int dv_stored, int per_head, hipStream_t stream) {

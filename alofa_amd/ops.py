@@ -1827,3 +1827,59 @@ def rms_pair_sum(out: torch.Tensor, a: torch.Tensor, wa: torch.Tensor, sa: float
     if a.shape != out.shape or b.shape != out.shape or wa.shape[0] != h or wb.shape[0] != h:
         raise AlofaError("shape_mismatch", "two branches of the output's shape, one weight per channel each", f"out={tuple(out.shape)} a={tuple(a.shape)} b={tuple(b.shape)}")
     _call("alofa_rms_pair_sum", _ptr(out), _ptr(a), _ptr(wa), _F(sa), _ptr(b), _ptr(wb), _F(sb), _L(T), _I(h), _F(eps), _I(int(exact)), _stream())
+
+
+def span_attention_fast(d: int, block_size: int, dtype) -> bool:
+    """Whether ``span_attention_mfma`` takes heads of d channels over pages of ``block_size`` tokens in this dtype."""
+    return dtype is torch.bfloat16 and d % 16 == 0 and 16 <= d <= MAX_HEAD_DIM and block_size >= MIN_FAST_PAGE and block_size & (block_size - 1) == 0
+
+
+def span_attention_mfma(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_table: torch.Tensor, tiles: Optional[torch.Tensor],
+                        req_of_token: Optional[torch.Tensor], positions: torch.Tensor, heads: int, kv_heads: int, d: int, window: Optional[int], scale: float,
+                        pooled: Optional[tuple] = None, bias: Optional[torch.Tensor] = None, sink: Optional[torch.Tensor] = None, gate: Optional[torch.Tensor] = None,
+                        gate_kind: int = GATE_NONE, dv_true: Optional[int] = None) -> None:
+    """``span_attention`` on the matrix cores, bfloat16: heads of d channels for keys and values alike (``dv_true`` of the value channels are the design's: the gate
+    per channel is [T, heads * dv_true]). ``tiles`` int32 [n, 3]: (request, first row, rows <= 16) of every run of rows that a wavefront serves per head; None: every
+    row is a run of its own (of request ``req_of_token[row]``, or of request ``row`` without it)."""
+    _gpu("out", out, torch.bfloat16, 2), _gpu("q", q, torch.bfloat16, 2), _gpu("k_cache", k_cache, torch.bfloat16, 4), _gpu("v_cache", v_cache, torch.bfloat16, 4)
+    _contig("k_cache", k_cache), _contig("v_cache", v_cache), _gpu("block_table", block_table, torch.int32, 2), _contig("block_table", block_table)
+    _gpu("positions", positions, torch.int32, 1), _contig("positions", positions)
+    T, block = q.shape[0], k_cache.shape[2]
+    dv_true = d if dv_true is None else int(dv_true)
+    if (tuple(q.shape) != (T, heads * d) or tuple(out.shape) != (T, heads * d) or tuple(k_cache.shape[1:]) != (kv_heads, block, d)
+            or tuple(v_cache.shape) != (k_cache.shape[0], kv_heads, d, block) or positions.shape[0] != T or not span_attention_fast(d, block, q.dtype)):
+        raise AlofaError("shape_mismatch", "attention operands do not fit the matrix-core kernel", f"out={tuple(out.shape)} q={tuple(q.shape)} k={tuple(k_cache.shape)} v={tuple(v_cache.shape)} heads={heads} kv_heads={kv_heads} d={d}")
+    pk = pv = pool_table = None
+    pool = places = 0
+    if pooled is not None:
+        pk, pv, pool_table, pool = pooled
+        places = _pooled_operands(pk, pv, pool_table, k_cache, kv_heads, d, d, pool)
+        if not window:
+            raise AlofaError("invalid_argument", "pooled blocks lie behind a window")
+    n_tiles = T
+    if tiles is not None:
+        _gpu("tiles", tiles, torch.int32, 2), _contig("tiles", tiles)
+        if tiles.shape[1] != 3:
+            raise AlofaError("shape_mismatch", "tiles are [n, 3]", f"tiles={tuple(tiles.shape)}")
+        n_tiles = tiles.shape[0]
+    elif req_of_token is not None:
+        _gpu("req_of_token", req_of_token, torch.int32, 1), _contig("req_of_token", req_of_token)
+    elif block_table.shape[0] < T or (pool_table is not None and pool_table.shape[0] < T):
+        raise AlofaError("shape_mismatch", "without a request per row every row is a request of its own", f"rows={T} tables={block_table.shape[0]}")
+    if bias is not None:
+        _gpu("bias", bias, torch.float32, 2), _contig("bias", bias)
+        if bias.shape[0] != heads or bias.shape[1] < 1:
+            raise AlofaError("shape_mismatch", "the bias is [heads, distances]", f"bias={tuple(bias.shape)}")
+    if sink is not None:
+        _gpu("sink", sink, torch.float32, 1), _contig("sink", sink)
+        if sink.shape[0] != heads:
+            raise AlofaError("shape_mismatch", "one sink per head", f"sink={tuple(sink.shape)}")
+    if gate_kind != GATE_NONE:
+        _gpu("gate", gate, torch.bfloat16, 2)
+        if tuple(gate.shape) != (T, heads * dv_true if gate_kind == GATE_CHANNEL else heads):
+            raise AlofaError("shape_mismatch", "the gate does not fit its kind", f"gate={tuple(gate.shape)} kind={gate_kind}")
+    _call("alofa_span_attention_mfma", _ptr(out), _L(_rows("out", out)), _ptr(q), _L(_rows("q", q)), _ptr(k_cache), _ptr(v_cache), _ptr(pk), _ptr(pv), _ptr(tiles), _I(n_tiles),
+          _ptr(block_table), _I(block_table.shape[1]), _ptr(pool_table), _I(pool_table.shape[1] if pool_table is not None else 0), _ptr(req_of_token), _ptr(positions),
+          _I(heads), _I(kv_heads), _I(d), _I(dv_true), _I(block), _I(int(window or 0)), _I(int(pool)), _I(places), _F(scale), _ptr(bias),
+          _I(bias.shape[1] if bias is not None else 0), _ptr(sink), _ptr(gate if gate_kind != GATE_NONE else None),
+          _L(_rows("gate", gate) if gate_kind != GATE_NONE else 0), _I(gate_kind), _stream())

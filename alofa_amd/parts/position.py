@@ -67,8 +67,12 @@ class Rotary(PositionEncoding):
                 inv[i] = inv[i] / np.float32(self.factor)
         ang = np.arange(n_positions, dtype=np.float32)[:, None] * inv[None, :]
         ang = ang.astype(np.float32).astype(np.float64)
-        mag = 1.0 if self.stretch is None else 0.1 * math.log(self.stretch["factor"]) + 1.0
-        return (np.cos(ang) * mag).astype(np.float32), (np.sin(ang) * mag).astype(np.float32)
+        cos, sin = np.cos(ang), np.sin(ang)
+        if self.stretch is not None:      # (the pairs that are turned grow; the channels that pass stay as they are)
+            mag = 0.1 * math.log(self.stretch["factor"]) + 1.0
+            cos[:, :self.dims // 2] *= mag
+            sin[:, :self.dims // 2] *= mag
+        return cos.astype(np.float32), sin.astype(np.float32)
 
     def _frequency(self, i: int) -> float:
         """Pair i's frequency in float64, with the linear factor and the stretch by wavelength."""

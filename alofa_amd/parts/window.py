@@ -25,6 +25,7 @@ value size are widened with zero rows to one size d, so that the matrix-core ker
 from __future__ import annotations
 
 import math
+import os
 
 import torch
 
@@ -35,6 +36,15 @@ from .attention import GQAAttention, RowPlan, _padded_heads
 from .base import SLOT, CacheNeed, CacheTensor, Mixer, build_part, part_class, register_part
 
 NAMES = {"q": "q", "k": "k", "v": "v", "o": "o", "gate": "g", "q_norm": "q.norm", "k_norm": "k.norm", "bias": "rel", "sink": "sink"}
+
+
+USE_SPAN_MFMA = os.environ.get("ALOFA_SPAN_MFMA", "1") != "0"      # 0 (for measurements): pooled blocks, bias and sink go through the always-valid kernel in bfloat16 too
+
+
+def _runs_of_sixteen(ctx) -> torch.Tensor:
+    """The step's rows as runs of up to sixteen rows of one request: int32 [n, 3] (request index, first row, rows)."""
+    runs = [(i, s.row0 + q0, min(16, s.n - q0)) for i, s in enumerate(ctx.spans) for q0 in range(0, s.n, 16)]
+    return torch.tensor(runs, dtype=torch.int32, device=ctx.device)
 
 
 def distance_buckets(rows: int, far: float, upto: int) -> list:
@@ -175,6 +185,26 @@ class WindowAttention(Mixer):
         if self.position is not None:
             self.position.table(n_positions)
 
+    def _plain_on_matrix_cores(self, ctx, kc) -> bool:
+        page = kc.shape[2]
+        if self.pooled is not None or self.bias is not None or self.sink is not None or self.rt.exact or self.rt.dtype is not torch.bfloat16:
+            return False
+        plan = ctx.memo("gqa_attention.rows", lambda: RowPlan(ctx))
+        return self.d % 16 == 0 and page >= ops.MIN_FAST_PAGE and page & (page - 1) == 0 and (plan.long_runs is None or self.d in ops.PREFILL_HEAD_DIMS)
+
+    def _attend_plain(self, ctx, q, kv, attn) -> None:
+        plan = ctx.memo("gqa_attention.rows", lambda: RowPlan(ctx))
+        common = (self.heads, self.kv_heads, self.d, self.window, self.scale)
+        if plan.long_runs is not None:
+            tiles, share, rows = plan.tiles(self.heads, self.kv_heads, self.d, self.window)
+            ops.attention_prefill(attn, q, kv.k, kv.v, kv.block_table, tiles, *common, share=share, rows=rows)
+        if plan.n_short:
+            floats = ops.decode_scratch_floats(plan.n_short, self.heads, self.kv_heads, self.d, ctx.max_context, self.window)
+            partial = ctx.scratch("attn_partial", (floats,), torch.float32) if floats else None
+            one_each = ctx.max_q_len == 1 and plan.short_rows is None and plan.long_runs is None
+            ops.attention_decode(attn, q, kv.k, kv.v, kv.block_table, None if one_each else ctx.req_of_token, ctx.positions, *common,
+                                 ctx.max_context, partial, rows=plan.short_rows)
+
     def forward(self, ctx, where, x, residual, out=None):
         T, exact = residual.shape[0], self.rt.exact
         entry, k = where if isinstance(where, tuple) else (where, 0)
@@ -194,7 +224,18 @@ class WindowAttention(Mixer):
             ops.pool_blocks(kv.k, kv.v, pooled[0], pooled[1], kv.block_table, pages.block_table, ctx.req_of_token, ctx.positions, G, D, D, int(self.pool), exact)
         attn = ctx.scratch("window_out", (T, H * D), self.rt.dtype)
         gate = proj[:, self.qkv_width:self.qkv_width + self.gate_width] if self.gate_kind is not None else None
-        if D != self.v_dim and gate is not None and self.gate_kind == "channel":
+        if self._plain_on_matrix_cores(ctx, kv.k):
+            # a window and nothing else: the engine's matrix-core kernels, portions of prompts and single tokens each by its own
+            self._attend_plain(ctx, proj[:, :H * D], kv, attn)
+            if gate is not None:
+                ops.head_gate(attn, gate, H, self.v_dim, self.gate_kind == "head", dv_stored=D)
+        elif not exact and USE_SPAN_MFMA and ops.span_attention_fast(D, kv.k.shape[2], self.rt.dtype):
+            # pooled blocks, a bias or a sink: this part's own matrix-core kernel, a wavefront per run of sixteen rows and head
+            tiles = None if ctx.max_q_len == 1 else ctx.memo("window_attention.runs", lambda: _runs_of_sixteen(ctx))
+            kind = ops.GATE_NONE if gate is None else (ops.GATE_CHANNEL if self.gate_kind == "channel" else ops.GATE_HEAD)
+            ops.span_attention_mfma(attn, proj[:, :H * D], kv.k, kv.v, kv.block_table, tiles, ctx.req_of_token, ctx.positions, H, G, D, self.window, self.scale,
+                                    pooled=pooled, bias=self.bias, sink=self.sink, gate=gate, gate_kind=kind, dv_true=self.v_dim)
+        elif D != self.v_dim and gate is not None and self.gate_kind == "channel":
             # (a gate per channel of the design's value heads against outputs of widened heads: applied afterwards, head by head)
             ops.span_attention(attn, proj[:, :H * D], kv.k, kv.v, kv.block_table, ctx.req_of_token, ctx.positions, H, G, D, D, self.window, self.scale, exact,
                                pooled=pooled, bias=self.bias, sink=self.sink)

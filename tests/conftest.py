@@ -127,3 +127,16 @@ def retotar_dirs(tmp_path_factory):
         write_random_model(cfg, d, seed=11 if name == "F" else 4000 + ord(name))
         out[name] = d
     return out
+
+
+@pytest.fixture(scope="session")
+def ludelorn_dirs(tmp_path_factory):
+    """Model folders of the small Ludelorn configurations, written by the engine's random-weights mode."""
+    from alofa_amd.weights import write_random_model
+    from ludelorn_cases import LUDELORN
+    out = {}
+    for name, cfg in LUDELORN.items():
+        d = tmp_path_factory.mktemp(f"ludelorn_{name}")
+        write_random_model(cfg, d, seed=5000 + ord(name))
+        out[name] = d
+    return out

@@ -125,10 +125,12 @@ def windowed_attention(h, W, m, eps, store=_id):
 
 def pooled_attention(h, W, m, eps, store=_id):
     """The mixer "attention": RMS norm over the whole query and key projections, rotation of neighbouring channels, a window,
-    and behind the window one mean key and mean value per whole block of ``pool`` tokens; tokens and blocks in one softmax."""
+    and behind the window one mean key and mean value per whole block of ``pool`` tokens (where the layer has blocks); tokens and
+    blocks in one softmax."""
     T = h.shape[0]
     H, G, d, dv = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
-    size, P = m["mask"]["size"], m["mask"]["pool"]
+    size = m["mask"]["size"]
+    P = m["mask"].get("pool") or T + 1      # (no blocks: none is ever whole)
     pos = torch.arange(T)
     q = rms(store(h @ W["q"].to(F).T), eps) * W["q.norm"].to(F)
     k = rms(store(h @ W["k"].to(F).T), eps) * W["k.norm"].to(F)
@@ -252,3 +254,38 @@ def forward(cfg, weights, tokens, store=_id, layers_out=None):
         if layers_out is not None:
             layers_out.append(x.clone())
     return store(rms(x, eps) * weights["final.norm"].to(F)) @ weights["head"].to(F).T
+
+
+# ---------------------------------------------------------------- for the tests
+
+def read_config(model_dir):
+    import json
+    from pathlib import Path
+    return json.loads((Path(model_dir) / "config.json").read_text())
+
+
+def read_weights(model_dir):
+    from pathlib import Path
+    from safetensors.torch import load_file
+    return {k: v.to(F) for k, v in load_file(str(Path(model_dir) / "model.safetensors")).items()}
+
+
+def to_bfloat16(x):
+    return x.to(torch.bfloat16).to(F)
+
+
+def forward_logits(weights, cfg, tokens, store=_id):
+    return forward(cfg, weights, tokens, store).numpy()
+
+
+def forward_hidden(weights, cfg, tokens):
+    out = []
+    forward(cfg, weights, tokens, layers_out=out)
+    return [x.numpy() for x in out]
+
+
+def greedy(weights, cfg, prompt, n_new):
+    ids = list(prompt)
+    for _ in range(n_new):
+        ids.append(int(forward(cfg, weights, ids)[-1].argmax()))
+    return ids[len(prompt):]
