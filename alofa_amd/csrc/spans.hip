@@ -277,7 +277,9 @@ __global__ void __launch_bounds__(256) span_attention_kernel(T* __restrict__ out
   }
 }
 
-// ---- the matrix-core kernel: a wavefront per (16 rows of one request, head), bfloat16 ---------------------------
+// ---- the matrix-core kernel: a block of four wavefronts per (16 rows of one request, head), bfloat16 ------------
+// The wavefronts take the tiles of keys in turn (a row's chain of dependent tiles is four times shorter) and their running states meet
+// in LDS at the end, combined in wavefront order.
 // Both products are taken transposed (v_mfma_f32_16x16x32_bf16; lane l: A row and B column l % 16, reduction slots 8 (l / 16) .. + 7,
 // D column l % 16 and rows 4 (l / 16) .. + 3), so a lane stays with one query row throughout:
 //   S^T[key, q] = K[key, :] . Q[q, :]       A = keys straight from the pages (16 bytes a lane), B = queries (registers)
@@ -313,9 +315,10 @@ __global__ void __launch_bounds__(256) span_attention_mfma_kernel(bf16_t* __rest
                                                                   const bf16_t* __restrict__ gate, SpanFastArgs a) {
   constexpr int d = DT * 16, DS = (d + 31) / 32;
   constexpr float kLow = -1e30f;
-  const int lane = threadIdx.x % kWave, col = lane % 16, grp = lane / 16;
-  const int h = blockIdx.y * 4 + threadIdx.x / kWave;
-  if (h >= a.heads) return;
+  __shared__ float others_acc[3][DT][kWave][4];      // what the wavefronts 1..3 hand to the first: their sums, ...
+  __shared__ float others_ml[3][2][kWave];           // ... maxima and weights' sums
+  const int lane = threadIdx.x % kWave, col = lane % 16, grp = lane / 16, wave = threadIdx.x / kWave;
+  const int h = blockIdx.y;
   const int g = h / (a.heads / a.kv_heads), S = 1 << a.bs_shift;
   int r, row0, n;
   if (a.tiles) {
@@ -373,7 +376,7 @@ __global__ void __launch_bounds__(256) span_attention_mfma_kernel(bf16_t* __rest
   };
 
   // ---- the window's tokens
-  for (int t0 = (lo / 32) * 32; t0 <= p_last; t0 += 32) {
+  for (int t0 = (lo / 32) * 32 + 32 * wave; t0 <= p_last; t0 += 128) {
     span_f32x4 sc[2];
     bool seen[2][4];
 #pragma unroll
@@ -425,7 +428,7 @@ __global__ void __launch_bounds__(256) span_attention_mfma_kernel(bf16_t* __rest
       page = ptab[first >> a.bs_shift];
       place = (first & (S - 1)) / a.P;
     };
-    for (int e0 = 0; e0 < n_blk_tile; e0 += 32) {
+    for (int e0 = 32 * wave; e0 < n_blk_tile; e0 += 128) {
       span_f32x4 sc[2];
       bool seen[2][4];
 #pragma unroll
@@ -465,6 +468,26 @@ __global__ void __launch_bounds__(256) span_attention_mfma_kernel(bf16_t* __rest
   }
 
   float total = rows_sum(l);
+  if (wave > 0) {
+    others_ml[wave - 1][0][lane] = m;
+    others_ml[wave - 1][1][lane] = total;
+#pragma unroll
+    for (int o = 0; o < DT; ++o)
+#pragma unroll
+      for (int x = 0; x < 4; ++x) others_acc[wave - 1][o][lane][x] = acc[o][x];
+  }
+  __syncthreads();
+  if (wave > 0) return;
+#pragma unroll
+  for (int w = 0; w < 3; ++w) {
+    const float m_w = others_ml[w][0][lane], m_new = fmaxf(m, m_w), mine = __expf(m - m_new), theirs = __expf(m_w - m_new);
+    total = total * mine + others_ml[w][1][lane] * theirs;
+    m = m_new;
+#pragma unroll
+    for (int o = 0; o < DT; ++o)
+#pragma unroll
+      for (int x = 0; x < 4; ++x) acc[o][x] = acc[o][x] * mine + others_acc[w][o][lane][x] * theirs;
+  }
   if (a.sink) {
     const float sk = a.sink[h], m_f = fmaxf(m, sk), alpha = __expf(m - m_f);
     total = total * alpha + __expf(sk - m_f);
@@ -602,7 +625,7 @@ extern "C" int alofa_span_attention_mfma(void* out, int64_t out_stride, const vo
   while ((1 << shift) < block_size) ++shift;
   SpanFastArgs a{out_stride, q_stride, gate_stride, tiles, table, max_blocks, pool_table, pool_max_blocks, req_of_token, positions, n_tiles, heads, kv_heads, shift, window,
                  P, places, dv_true, scale, bias, bias_len, sink, gate_kind};
-  const dim3 grid(n_tiles, (heads + 3) / 4);
+  const dim3 grid(n_tiles, heads);
   switch (d / 16) {
 #define ALOFA_SPAN_DT(N) case N: launch_span_mfma<N>(grid, stream, out, q, k_cache, v_cache, pk, pv, gate, a); break;
     ALOFA_SPAN_DT(1) ALOFA_SPAN_DT(2) ALOFA_SPAN_DT(3) ALOFA_SPAN_DT(4) ALOFA_SPAN_DT(5) ALOFA_SPAN_DT(6) ALOFA_SPAN_DT(7) ALOFA_SPAN_DT(8)

@@ -1883,3 +1883,56 @@ def span_attention_mfma(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tenso
           _I(heads), _I(kv_heads), _I(d), _I(dv_true), _I(block), _I(int(window or 0)), _I(int(pool)), _I(places), _F(scale), _ptr(bias),
           _I(bias.shape[1] if bias is not None else 0), _ptr(sink), _ptr(gate if gate_kind != GATE_NONE else None),
           _L(_rows("gate", gate) if gate_kind != GATE_NONE else 0), _I(gate_kind), _stream())
+
+
+def rms_pair_add_norm(residual: torch.Tensor, a: torch.Tensor, wa: torch.Tensor, sa: float, b: torch.Tensor, wb: torch.Tensor, sb: float, scale: Optional[torch.Tensor],
+                      eps: float, exact: bool = False, then_norm: Optional[tuple] = None) -> None:
+    """residual[t, c] += scale[c] * (sa * a[t] / rms(a[t]) * wa + sb * b[t] / rms(b[t]) * wb)[c] (``scale`` None: ones); with ``then_norm`` = (weight, eps, rows) the same
+    launch leaves rows[t] = rmsnorm(residual[t]) * weight."""
+    for n, t in (("residual", residual), ("a", a), ("b", b)):
+        _gpu(n, t, torch.float32, 2), _contig(n, t)
+    _gpu("wa", wa, torch.float32, 1), _gpu("wb", wb, torch.float32, 1), _contig("wa", wa), _contig("wb", wb)
+    T, h = residual.shape
+    if a.shape != residual.shape or b.shape != residual.shape or wa.shape[0] != h or wb.shape[0] != h:
+        raise AlofaError("shape_mismatch", "two branches of the stream's shape, one weight per channel each", f"residual={tuple(residual.shape)} a={tuple(a.shape)} b={tuple(b.shape)}")
+    if scale is not None:
+        _gpu("scale", scale, torch.float32, 1), _contig("scale", scale)
+        if scale.shape[0] != h:
+            raise AlofaError("shape_mismatch", "one factor per channel", f"scale={tuple(scale.shape)}")
+    nw = rows = None
+    norm_eps = 0.0
+    if then_norm is not None:
+        nw, norm_eps, rows = then_norm
+        _gpu("norm weight", nw, torch.float32, 1), _contig("norm weight", nw), _gpu("normed rows", rows, None, 2), _contig("normed rows", rows)
+        if nw.shape[0] != h or rows.shape != residual.shape:
+            raise AlofaError("shape_mismatch", "the norm behind the sum does not fit", f"weight={tuple(nw.shape)} rows={tuple(rows.shape)}")
+    _call("alofa_rms_pair_add_norm", _ptr(residual), _ptr(a), _ptr(wa), _F(sa), _ptr(b), _ptr(wb), _F(sb), _ptr(scale), _L(T), _I(h), _F(eps), _ptr(rows),
+          _I(dtype_code(rows) if rows is not None else F32), _ptr(nw), _F(norm_eps), _I(int(exact)), _stream())
+
+
+def ssd_step(xbc: torch.Tensor, raw: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], state: Optional[torch.Tensor], rows: RowsOfRequests, qf: torch.Tensor,
+             kf: torch.Tensor, vf: torch.Tensor, decay: torch.Tensor, dt_raw: torch.Tensor, dt_bias: torch.Tensor, a_log: torch.Tensor, heads: int, groups: int,
+             n_state: int, dv: int, exact: bool = False) -> None:
+    """``conv_bias_act`` (with silu), ``conv_keep`` and ``ssd_operands`` in one launch, for a step in which every request brings one row."""
+    T, width = raw.shape
+    taps = w.shape[1]
+    _gpu("xbc", xbc, raw.dtype, 2), _gpu("raw", raw, None, 2), _gpu("w", w, torch.float32, 2), _contig("w", w)
+    if rows.offsets is not None or rows.rows != T or tuple(xbc.shape) != (T, width) or width != heads * dv + 2 * groups * n_state or w.shape[0] != width or not 1 <= taps <= CONV_MAX_TAPS:
+        raise AlofaError("shape_mismatch", "one row per request, rows of x, B, C side by side", f"raw={tuple(raw.shape)} xbc={tuple(xbc.shape)} w={tuple(w.shape)} heads={heads} groups={groups}")
+    if taps > 1:
+        _gpu("state", state, raw.dtype, 3), _contig("state", state)
+        if tuple(state.shape[1:]) != (taps - 1, width):
+            raise AlofaError("shape_mismatch", "the convolution's state does not fit", f"state={tuple(state.shape)}")
+        rows.fits("state", state)
+    if bias is not None:
+        _gpu("bias", bias, torch.float32, 1), _contig("bias", bias)
+    for n, t, wd in (("qf", qf, heads * n_state), ("kf", kf, heads * n_state), ("decay", decay, heads * n_state), ("vf", vf, heads * dv)):
+        _gpu(n, t, torch.float32, 2), _contig(n, t)
+        if tuple(t.shape) != (T, wd):
+            raise AlofaError("shape_mismatch", "the float operands do not fit", f"operand={n} shape={tuple(t.shape)}")
+    _gpu("dt_raw", dt_raw, raw.dtype, 2), _gpu("dt_bias", dt_bias, torch.float32, 1), _gpu("a_log", a_log, torch.float32, 1), _contig("dt_bias", dt_bias), _contig("a_log", a_log)
+    if tuple(dt_raw.shape) != (T, heads) or dt_bias.shape[0] != heads or a_log.shape[0] != heads or (bias is not None and bias.shape[0] != width):
+        raise AlofaError("shape_mismatch", "one step size, bias and rate per head", f"dt={tuple(dt_raw.shape)}")
+    _call("alofa_ssd_step", _ptr(xbc), _L(_rows("xbc", xbc)), _ptr(raw), _L(_rows("raw", raw)), _I(dtype_code(raw)), _ptr(w), _ptr(bias), _ptr(state if taps > 1 else None),
+          _ptr(rows.slots), _I(taps), _ptr(qf), _ptr(kf), _ptr(vf), _ptr(decay), _ptr(dt_raw), _L(_rows("dt_raw", dt_raw)), _ptr(dt_bias), _ptr(a_log), _L(T), _I(heads),
+          _I(groups), _I(n_state), _I(dv), _I(int(exact)), _stream())

@@ -307,7 +307,7 @@ class StateSpace(RecurrentMixer):
                              f"heads={self.heads} groups={self.groups} norm_parts={self.norm_parts} taps={self.taps}")
         w_in = weights[pre + "in"]
         if w_in.shape[0] % 8:      # (rows of the projection stay 16-byte aligned)
-            w_in = torch.cat([w_in, torch.zeros((8 - w_in.shape[0] % 8, w_in.shape[1]), dtype=w_in.dtype)])
+            w_in = torch.cat([w_in, torch.zeros((8 - w_in.shape[0] % 8, w_in.shape[1]), dtype=w_in.dtype, device=w_in.device)])
         self.w_in, self.w_o = rt.matrix(w_in), rt.matrix(weights[pre + "o"])
         self.conv_w, self.conv_b = rt.vector(weights[pre + "conv"]), rt.vector(weights[pre + "conv.b"])
         self.dt_bias, self.a_log, self.skip = rt.vector(weights[pre + "dt_bias"]), rt.vector(weights[pre + "A_log"]), rt.vector(weights[pre + "D"])
@@ -325,16 +325,19 @@ class StateSpace(RecurrentMixer):
         ops.gemm(proj, x, self.w_in, exact=exact)
         z, raw, dt = proj[:, :inner], proj[:, inner:inner + self.conv_width], proj[:, inner + self.conv_width:inner + self.conv_width + H]
         xbc = ctx.scratch("state_space_conv", (T, self.conv_width), self.rt.dtype)
-        if self.taps > 1:
-            tail = ctx.state((entry, k + 1))
-            ops.conv_bias_act(xbc, raw, self.conv_w, self.conv_b, tail, rows, silu=True, exact=exact)
-            ops.conv_keep(tail, raw, rows)
-        else:
-            none = ctx.scratch("conv_no_state", (ctx.fn.cache.max_requests, 0, self.conv_width), self.rt.dtype)
-            ops.conv_bias_act(xbc, raw, self.conv_w, self.conv_b, none, rows, silu=True, exact=exact)
         qf, kf = ctx.scratch("memory_q", (T, H * N), torch.float32), ctx.scratch("memory_k", (T, H * N), torch.float32)
         vf, decay = ctx.scratch("memory_v", (T, inner), torch.float32), ctx.scratch("recurrent_decay", (T, H * N), torch.float32)
-        ops.ssd_operands(qf, kf, vf, decay, xbc, dt, self.dt_bias, self.a_log, H, self.groups, N, dv, exact)
+        tail = ctx.state((entry, k + 1)) if self.taps > 1 else None
+        if rows.offsets is None:      # single rows (decoding): the convolution, its state's step and the operands are one launch
+            ops.ssd_step(xbc, raw, self.conv_w, self.conv_b, tail, rows, qf, kf, vf, decay, dt, self.dt_bias, self.a_log, H, self.groups, N, dv, exact)
+        else:
+            if tail is not None:
+                ops.conv_bias_act(xbc, raw, self.conv_w, self.conv_b, tail, rows, silu=True, exact=exact)
+                ops.conv_keep(tail, raw, rows)
+            else:
+                none = ctx.scratch("conv_no_state", (ctx.fn.cache.max_requests, 0, self.conv_width), self.rt.dtype)
+                ops.conv_bias_act(xbc, raw, self.conv_w, self.conv_b, none, rows, silu=True, exact=exact)
+            ops.ssd_operands(qf, kf, vf, decay, xbc, dt, self.dt_bias, self.a_log, H, self.groups, N, dv, exact)
         o = self._readouts(ctx, T)
         parts = ops.linear_recurrence(o, qf, kf, vf, ctx.state((entry, k)), rows, H, N, dv, ops.DECAY_GIVEN, decay)
         y = ctx.scratch("recurrent_gated", (T, inner), self.rt.dtype)
@@ -467,7 +470,12 @@ class ParallelMixers(Mixer):
         for b in self.branches:
             b.prepare(n_positions)
 
-    def forward(self, ctx, where, x, residual, out=None):
+    @property
+    def takes_channel_scale(self):
+        """Normed branches join the stream in a launch of their own, which also applies a factor per channel (``scale=``) and leaves the next norm (``then=``)."""
+        return bool(self.norms)
+
+    def forward(self, ctx, where, x, residual, out=None, scale=None, then=None):
         entry, k = where if isinstance(where, tuple) else (where, 0)
         outs = []
         for j, b in enumerate(self.branches):
@@ -479,8 +487,7 @@ class ParallelMixers(Mixer):
             if out is not None:
                 ops.rms_pair_sum(out, outs[0], self.norms[0], self.scales[0], outs[1], self.norms[1], self.scales[1], self.eps, self.rt.exact)
             else:
-                ops.rms_pair_sum(outs[0], outs[0], self.norms[0], self.scales[0], outs[1], self.norms[1], self.scales[1], self.eps, self.rt.exact)
-                ops.add_scaled(residual, outs[0], 1.0, exact=self.rt.exact)
+                ops.rms_pair_add_norm(residual, outs[0], self.norms[0], self.scales[0], outs[1], self.norms[1], self.scales[1], scale, self.eps, self.rt.exact, then_norm=then)
             return
         target = residual
         if out is not None:

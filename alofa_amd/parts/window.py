@@ -142,7 +142,7 @@ class WindowAttention(Mixer):
             self.gate_width = mats[-1].shape[0]
         rows = self.qkv_width + self.gate_width
         if rows % 8:      # (rows of the projection stay 16-byte aligned)
-            mats.append(torch.zeros((8 - rows % 8, self.hidden), dtype=mats[0].dtype))
+            mats.append(torch.zeros((8 - rows % 8, self.hidden), dtype=mats[0].dtype, device=mats[0].device))
         if len({m.dtype for m in mats}) > 1:
             mats = [m.float() for m in mats]
         self.w_in = rt.matrix(torch.cat(mats, dim=0))
@@ -169,7 +169,7 @@ class WindowAttention(Mixer):
                 raise AlofaError("invalid_argument", "the bias table has at least two rows and reaches beyond its evenly spaced half", f"rows={rows_n} far={far}")
             # every distance the window lets through has its row; beyond ``far`` all distances share the last one
             upto = int(math.ceil(far)) + 1 if self.window is None else min(int(self.window), int(math.ceil(far)) + 1)
-            self.bias = rt.vector(table[torch.tensor(distance_buckets(rows_n, far, upto))].t().contiguous())      # [heads, distances]
+            self.bias = rt.vector(table[torch.tensor(distance_buckets(rows_n, far, upto), device=table.device)].t().contiguous())      # [heads, distances]
         self.sink = rt.vector(weights[pre + n["sink"]]) if p.get("sink", False) else None
         self.pooled = PooledBlocks(G, D, int(self.pool), rt) if self.pool is not None else None
         # the pages are kept as long as a block that a row completes can still be read whole

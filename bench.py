@@ -28,7 +28,7 @@ context of 4,096) through the same engine and print their own line;
 ``--config 1.5b``, ``3b`` and ``14b`` run the continuous batch at those sizes.
 ``--sweep batch`` and ``--sweep context`` take any of the configurations.
 
-``--design tugalix``, ``--design rerupel`` and ``--design retotar`` measure another design beside Qwen2 (Retotar: beside Tugalix) at equal sizes: prefill of one prompt and
+``--design tugalix``, ``--design rerupel``, ``--design retotar`` and ``--design ludelorn`` measure another design beside Qwen2 (Retotar and Ludelorn: beside Tugalix) at equal sizes: prefill of one prompt and
 decode steps at batch 1, 8 and 64, at a few widths (``--sizes``), a line per point and model."""
 import argparse
 import json
@@ -549,8 +549,26 @@ def retotar_sizes(width, heads, dim, ff, layers, vocab=32000):
     return ret, tugalix_sizes(width, heads, dim, 6 * expert, layers, vocab)[0]
 
 
-DESIGN_MODELS = {"tugalix": tugalix_sizes, "rerupel": rerupel_sizes, "retotar": retotar_sizes}
-DESIGN_BESIDE = {"retotar": "tugalix"}      # the model a design is measured beside, where that is not Qwen2
+def ludelorn_sizes(width, heads, dim, ff, layers, vocab=32000):
+    """A Ludelorn model of ``layers`` layers in the order parallel (attention within 1,024 keys beside a state-space mixer of as many heads,
+    state channels as a head has channels), attention within 512 keys with pooled blocks of 16 behind them, parallel, attention with a bias
+    by distance and a sink within 512 keys, every one with a dense feed-forward, and beside it the closest other design, Tugalix (attention
+    beside a recurrence, dense feed-forwards), at equal width, heads, layers and feed-forward."""
+    kv = max(1, heads // 4)
+    left = {"heads": heads, "kv_heads": kv, "dim": dim, "vdim": dim, "scale": dim ** -0.5, "mask": {"size": 1024},
+            "rot": {"dims": dim, "base": 1000000.0, "scaling": {"factor": 4.0, "original": 4096, "fast": 32.0, "slow": 1.0}}}
+    right = {"heads": heads, "vdim": dim, "state": dim, "groups": max(1, heads // 8), "conv": 4, "norm_groups": max(1, heads // 8)}
+    kinds = [("parallel", {"left": left, "right": right}),
+             ("attention", {"heads": heads, "kv_heads": kv, "dim": dim, "vdim": dim, "scale": dim ** -0.5, "mask": {"size": 512, "pool": 16}, "rot": {"dims": dim // 2, "base": 500000.0}}),
+             ("parallel", {"left": left, "right": right}),
+             ("attention_2", {"heads": heads, "kv_heads": kv, "dim": dim, "vdim": dim, "scale": 8.0 / dim, "mask": {"size": 512}, "bias_max": 512.0, "bias_rows": 32})]
+    lud = {"architecture": "Ludelorn", "vocab": vocab, "width": width, "norm": {"eps": 1e-6}, "embedding": {"scale": 1.0},
+           "layers": [{"type": kinds[i % 4][0], "mixer": kinds[i % 4][1], "mlp": {"kind": "dense", "ff": ff}} for i in range(layers)]}
+    return lud, tugalix_sizes(width, heads, dim, ff, layers, vocab)[0]
+
+
+DESIGN_MODELS = {"tugalix": tugalix_sizes, "rerupel": rerupel_sizes, "retotar": retotar_sizes, "ludelorn": ludelorn_sizes}
+DESIGN_BESIDE = {"retotar": "tugalix", "ludelorn": "tugalix"}      # the model a design is measured beside, where that is not Qwen2
 DESIGN_SIZES = {"256": (256, 4, 64, 1024, 4), "1k": (1024, 16, 64, 4096, 8), "2k": (2048, 16, 128, 8192, 8), "4k": (4096, 32, 128, 14336, 4)}
 DESIGN_DEFAULT = ("1k", "2k", "4k")      # ("256": a small one, for a quick look)
 
