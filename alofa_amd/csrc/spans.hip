@@ -28,19 +28,18 @@ enum NormScope : int { kNormNone = 0, kNormHead = 1, kNormAll = 2 };
 // The mean is taken over q_count and k_count channels (heads that were widened with zeros hold fewer than their width).
 template <typename T, typename Acc>
 __global__ void __launch_bounds__(256) projection_inv_rms_kernel(double* __restrict__ inv, const T* __restrict__ qkv, int64_t stride, int tokens, int q_width, int k_width, int q_count, int k_count, float eps) {
-  const int64_t unit = static_cast<int64_t>(blockIdx.x) * 4 + threadIdx.x / kWave;
-  if (unit >= 2 * static_cast<int64_t>(tokens)) return;
-  const int lane = threadIdx.x % kWave;
-  const int t = static_cast<int>(unit / 2), which = static_cast<int>(unit % 2);
+  __shared__ Acc scratch[4];
+  const int unit = blockIdx.x;      // (a block per row and projection)
+  const int t = unit / 2, which = unit % 2;
   const T* x = qkv + static_cast<int64_t>(t) * stride + (which ? q_width : 0);
   const int n = which ? k_width : q_width;
   Acc ss = 0;
-  for (int c = lane; c < n; c += kWave) {
+  for (int c = threadIdx.x; c < n; c += 256) {
     const Acc v = static_cast<Acc>(load_f32(x + c));
     ss += v * v;
   }
-  ss = wave_sum(ss);
-  if (lane == 0) inv[unit] = static_cast<double>(static_cast<Acc>(1) / sqrt(ss / static_cast<Acc>(which ? k_count : q_count) + static_cast<Acc>(eps)));
+  ss = block_sum<Acc, 256>(ss, scratch);
+  if (threadIdx.x == 0) inv[unit] = static_cast<double>(static_cast<Acc>(1) / sqrt(ss / static_cast<Acc>(which ? k_count : q_count) + static_cast<Acc>(eps)));
 }
 
 // One wavefront per (row, unit): query heads first, then key heads, then (unless the values are the keys) value heads.
@@ -277,8 +276,8 @@ __global__ void __launch_bounds__(256) span_attention_kernel(T* __restrict__ out
   }
 }
 
-// ---- the matrix-core kernel: a block of four wavefronts per (16 rows of one request, head), bfloat16 ------------
-// The wavefronts take the tiles of keys in turn (a row's chain of dependent tiles is four times shorter) and their running states meet
+// ---- the matrix-core kernel: a block of four or eight wavefronts per (16 rows of one request, head), bfloat16
+// The wavefronts take the tiles of keys in turn (a row's chain of dependent tiles is as many times shorter) and their running states meet
 // in LDS at the end, combined in wavefront order.
 // Both products are taken transposed (v_mfma_f32_16x16x32_bf16; lane l: A row and B column l % 16, reduction slots 8 (l / 16) .. + 7,
 // D column l % 16 and rows 4 (l / 16) .. + 3), so a lane stays with one query row throughout:
@@ -288,7 +287,8 @@ __global__ void __launch_bounds__(256) span_attention_kernel(T* __restrict__ out
 // keys 4 g + r and 16 + 4 g + r (g = l / 16, r = 0..3), which are the eight reduction slots of the second product when the values are read
 // in that order, so the weights never leave their registers. The four lanes of a query meet for the tile's maximum; the running
 // maximum, the weights' sum and the scores are float. Then the blocks behind the window, 32 at a time, the same way (their places
-// are looked up one by one). The sink joins the denominator at the end; the gate rides on the store.
+// are looked up one by one). The sink joins the denominator at the end; the gate rides on the store. Every weight enters the second
+// product as two bfloat16 numbers (sixteen bits of it count).
 typedef __bf16 span_bf16x8 __attribute__((ext_vector_type(8)));
 typedef float span_f32x4 __attribute__((ext_vector_type(4)));
 
@@ -309,14 +309,14 @@ struct SpanFastArgs {
   int gate_kind;
 };
 
-template <int DT>
-__global__ void __launch_bounds__(256) span_attention_mfma_kernel(bf16_t* __restrict__ out, const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_cache,
+template <int DT, int NW>
+__global__ void __launch_bounds__(64 * NW) span_attention_mfma_kernel(bf16_t* __restrict__ out, const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_cache,
                                                                   const bf16_t* __restrict__ v_cache, const bf16_t* __restrict__ pk, const bf16_t* __restrict__ pv,
                                                                   const bf16_t* __restrict__ gate, SpanFastArgs a) {
   constexpr int d = DT * 16, DS = (d + 31) / 32;
   constexpr float kLow = -1e30f;
-  __shared__ float others_acc[3][DT][kWave][4];      // what the wavefronts 1..3 hand to the first: their sums, ...
-  __shared__ float others_ml[3][2][kWave];           // ... maxima and weights' sums
+  __shared__ float others_acc[NW - 1][DT][kWave][4];      // what the other wavefronts hand to the first: their sums, ...
+  __shared__ float others_ml[NW - 1][2][kWave];           // ... maxima and weights' sums
   const int lane = threadIdx.x % kWave, col = lane % 16, grp = lane / 16, wave = threadIdx.x / kWave;
   const int h = blockIdx.y;
   const int g = h / (a.heads / a.kv_heads), S = 1 << a.bs_shift;
@@ -356,7 +356,8 @@ __global__ void __launch_bounds__(256) span_attention_mfma_kernel(bf16_t* __rest
       for (int x = 0; x < 4; ++x) top = fmaxf(top, seen[u][x] ? sc[u][x] : kLow);
     top = rows_max(top);
     const float m_new = fmaxf(m, top), alpha = __expf(m - m_new);
-    span_bf16x8 w;
+    // (the weights are 32-bit numbers: each meets the values as two bfloat16 numbers, its rounding and what the rounding took away)
+    span_bf16x8 w, rest;
     float sum = 0.f;
 #pragma unroll
     for (int u = 0; u < 2; ++u)
@@ -365,18 +366,21 @@ __global__ void __launch_bounds__(256) span_attention_mfma_kernel(bf16_t* __rest
         const float e = seen[u][x] ? __expf(sc[u][x] - m_new) : 0.f;
         sum += e;
         w[4 * u + x] = static_cast<__bf16>(e);
+        rest[4 * u + x] = static_cast<__bf16>(e - static_cast<float>(w[4 * u + x]));
       }
     l = l * alpha + sum;
     m = m_new;
 #pragma unroll
     for (int o = 0; o < DT; ++o) {
+      const span_bf16x8 vf = values(o);
       acc[o] *= alpha;
-      acc[o] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(values(o), w, acc[o], 0, 0, 0);
+      acc[o] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, w, acc[o], 0, 0, 0);
+      acc[o] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, rest, acc[o], 0, 0, 0);
     }
   };
 
   // ---- the window's tokens
-  for (int t0 = (lo / 32) * 32 + 32 * wave; t0 <= p_last; t0 += 128) {
+  for (int t0 = (lo / 32) * 32 + 32 * wave; t0 <= p_last; t0 += 32 * NW) {
     span_f32x4 sc[2];
     bool seen[2][4];
 #pragma unroll
@@ -428,7 +432,7 @@ __global__ void __launch_bounds__(256) span_attention_mfma_kernel(bf16_t* __rest
       page = ptab[first >> a.bs_shift];
       place = (first & (S - 1)) / a.P;
     };
-    for (int e0 = 32 * wave; e0 < n_blk_tile; e0 += 128) {
+    for (int e0 = 32 * wave; e0 < n_blk_tile; e0 += 32 * NW) {
       span_f32x4 sc[2];
       bool seen[2][4];
 #pragma unroll
@@ -479,7 +483,7 @@ __global__ void __launch_bounds__(256) span_attention_mfma_kernel(bf16_t* __rest
   __syncthreads();
   if (wave > 0) return;
 #pragma unroll
-  for (int w = 0; w < 3; ++w) {
+  for (int w = 0; w < NW - 1; ++w) {
     const float m_w = others_ml[w][0][lane], m_new = fmaxf(m, m_w), mine = __expf(m - m_new), theirs = __expf(m_w - m_new);
     total = total * mine + others_ml[w][1][lane] * theirs;
     m = m_new;
@@ -545,7 +549,7 @@ extern "C" int alofa_norm_turn_write(void* qkv, int64_t stride, int dtype, const
   const int per_row = heads + kv_heads + (values_are_keys ? 0 : kv_heads);
   ALOFA_REQUIRE(scope != kNormAll || row_inv != nullptr, "norm_turn_write: a norm over the whole projection needs room for the rows' factors");
   if (scope == kNormAll) {
-    const unsigned g2 = static_cast<unsigned>((2 * static_cast<int64_t>(tokens) + 3) / 4);
+    const unsigned g2 = static_cast<unsigned>(2 * static_cast<int64_t>(tokens));
     if (exact) projection_inv_rms_kernel<float, double><<<g2, 256, 0, stream>>>(row_inv, static_cast<const float*>(qkv), stride, tokens, heads * d, kv_heads * d, heads * d_true, kv_heads * d_true, eps);
     else if (dtype == kF32) projection_inv_rms_kernel<float, float><<<g2, 256, 0, stream>>>(row_inv, static_cast<const float*>(qkv), stride, tokens, heads * d, kv_heads * d, heads * d_true, kv_heads * d_true, eps);
     else projection_inv_rms_kernel<bf16_t, float><<<g2, 256, 0, stream>>>(row_inv, static_cast<const bf16_t*>(qkv), stride, tokens, heads * d, kv_heads * d, heads * d_true, kv_heads * d_true, eps);
@@ -603,8 +607,13 @@ extern "C" int alofa_span_attention(void* out, int64_t out_stride, const void* q
 template <int DT>
 static void launch_span_mfma(dim3 grid, hipStream_t stream, void* out, const void* q, const void* k_cache, const void* v_cache, const void* pk, const void* pv, const void* gate,
                              const SpanFastArgs& a) {
-  span_attention_mfma_kernel<DT><<<grid, 256, 0, stream>>>(static_cast<bf16_t*>(out), static_cast<const bf16_t*>(q), static_cast<const bf16_t*>(k_cache), static_cast<const bf16_t*>(v_cache),
-                                                           static_cast<const bf16_t*>(pk), static_cast<const bf16_t*>(pv), static_cast<const bf16_t*>(gate), a);
+  // (single rows, where blocks are few: eight wavefronts where their states fit the LDS a block may name; runs of rows: four, 78 against 91 us a layer of a 2,048-token prompt)
+  if (DT <= 8 && a.tiles == nullptr)
+    span_attention_mfma_kernel<DT, (DT <= 8 ? 8 : 4)><<<grid, 64 * 8, 0, stream>>>(static_cast<bf16_t*>(out), static_cast<const bf16_t*>(q), static_cast<const bf16_t*>(k_cache), static_cast<const bf16_t*>(v_cache),
+                                                                            static_cast<const bf16_t*>(pk), static_cast<const bf16_t*>(pv), static_cast<const bf16_t*>(gate), a);
+  else
+    span_attention_mfma_kernel<DT, 4><<<grid, 256, 0, stream>>>(static_cast<bf16_t*>(out), static_cast<const bf16_t*>(q), static_cast<const bf16_t*>(k_cache), static_cast<const bf16_t*>(v_cache),
+                                                                static_cast<const bf16_t*>(pk), static_cast<const bf16_t*>(pv), static_cast<const bf16_t*>(gate), a);
 }
 
 // bfloat16 on the matrix cores: heads of d = dv channels in steps of 16, pages of a power of two of at least 8 tokens, rows 16-byte aligned.

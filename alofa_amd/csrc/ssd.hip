@@ -6,7 +6,7 @@
 //   ssd_operands      the recurrence's operands as float32 rows: step size dt = softplus(z + bias) per head, decay
 //                     exp(-exp(A_log) dt), keys dt * B and queries C of the head's group, values x.
 //   ssd_finish        y = (read-out + D x) * silu(z), an RMS norm over each of several equal parts of the row, a weight.
-//   ssd_step          conv_bias_act, the state's step and ssd_operands in one launch, for steps of single rows.
+//   ssd_step          for steps of single rows: conv_bias_act with the state's step in one launch, then ssd_operands.
 //   rms_pair_add_norm the sum of two normed branches into the stream, times a factor per channel, and the next norm, one launch.
 //   rms_pair_sum      out = sa * rms(a) * wa + sb * rms(b) * wb: two branches, each normed over the width, summed (out may be a or b:
 //                     a thread reads what it owns of a row before it writes there).
@@ -169,57 +169,31 @@ __global__ void __launch_bounds__(256) rms_pair_add_norm_kernel(float* __restric
   for (int c = threadIdx.x; c < width; c += 256) store_f32(normed + t * width + c, static_cast<float>(static_cast<Acc>(rr[c]) * inv * static_cast<Acc>(nw[c])));
 }
 
-// A step in which every request brings one row (row r is request r): the convolution with bias and silu, the state's step and the
-// recurrence's operands in one launch. A block per row: its threads first take the row's channels through the convolution (a thread
-// fetches what the state holds of its channel, then writes), then, once the row is whole, form the operands head by head.
+// A step in which every request brings one row (row r is request r): the convolution with bias and silu and the state's step in one
+// launch. A thread owns one channel of one row: it fetches what the state holds of its channel, then writes.
 template <typename T, typename Acc>
-__global__ void __launch_bounds__(256) ssd_step_kernel(T* __restrict__ xbc, int64_t xbc_stride, const T* __restrict__ raw, int64_t raw_stride, const float* __restrict__ w,
-                                                       const float* __restrict__ bias, T* __restrict__ state, const int32_t* __restrict__ req_slot, int taps,
-                                                       float* __restrict__ qf, float* __restrict__ kf, float* __restrict__ vf, float* __restrict__ decay,
-                                                       const T* __restrict__ dt_raw, int64_t dt_stride, const float* __restrict__ dt_bias, const float* __restrict__ a_log,
-                                                       int heads, int groups, int N, int dv) {
-  extern __shared__ double ssd_step_lds[];      // [heads] step sizes, [heads] decays (as Acc)
-  const int64_t t = blockIdx.x;
-  const int width = heads * dv + 2 * groups * N, keep = taps - 1;
+__global__ void __launch_bounds__(256) conv_step_kernel(T* __restrict__ xbc, int64_t xbc_stride, const T* __restrict__ raw, int64_t raw_stride, const float* __restrict__ w,
+                                                        const float* __restrict__ bias, T* __restrict__ state, const int32_t* __restrict__ req_slot, int width, int taps) {
+  const int64_t t = blockIdx.y;
+  const int c = blockIdx.x * 256 + threadIdx.x, keep = taps - 1;
+  if (c >= width) return;
   T* st = state + static_cast<int64_t>(req_slot[t]) * keep * width;
-  T* row = xbc + t * xbc_stride;
-  for (int c = threadIdx.x; c < width; c += 256) {
-    const float* wc = w + static_cast<int64_t>(c) * taps;
-    T kept[kConvMaxKeep];
-    Acc acc = bias ? static_cast<Acc>(bias[c]) : static_cast<Acc>(0);
+  const float* wc = w + static_cast<int64_t>(c) * taps;
+  T kept[kConvMaxKeep];
+  Acc acc = bias ? static_cast<Acc>(bias[c]) : static_cast<Acc>(0);
 #pragma unroll
-    for (int j = 0; j < kConvMaxKeep; ++j)
-      if (j < keep) {
-        kept[j] = st[static_cast<int64_t>(j) * width + c];
-        acc += static_cast<Acc>(wc[j]) * static_cast<Acc>(load_f32(&kept[j]));
-      }
-    const T mine = raw[t * raw_stride + c];
-    acc += static_cast<Acc>(wc[keep]) * static_cast<Acc>(load_f32(&mine));
+  for (int j = 0; j < kConvMaxKeep; ++j)
+    if (j < keep) {
+      kept[j] = st[static_cast<int64_t>(j) * width + c];
+      acc += static_cast<Acc>(wc[j]) * static_cast<Acc>(load_f32(&kept[j]));
+    }
+  const T mine = raw[t * raw_stride + c];
+  acc += static_cast<Acc>(wc[keep]) * static_cast<Acc>(load_f32(&mine));
 #pragma unroll
-    for (int j = 0; j < kConvMaxKeep; ++j)
-      if (j < keep) st[static_cast<int64_t>(j) * width + c] = j + 1 < keep ? kept[j + 1] : mine;
-    acc = acc / (static_cast<Acc>(1) + exp(-acc));
-    store_f32(row + c, static_cast<float>(acc));
-  }
-  Acc* steps = reinterpret_cast<Acc*>(ssd_step_lds);
-  Acc* keeps = steps + heads;
-  for (int h = threadIdx.x; h < heads; h += 256) {
-    const Acc z = static_cast<Acc>(load_f32(dt_raw + t * dt_stride + h)) + static_cast<Acc>(dt_bias[h]);
-    const Acc dt = (z > 0 ? z : static_cast<Acc>(0)) + log1p(exp(-fabs(z)));
-    steps[h] = dt;
-    keeps[h] = exp(-exp(static_cast<Acc>(a_log[h])) * dt);
-  }
-  __threadfence_block();
-  __syncthreads();
-  const int per = heads / groups;
-  for (int e = threadIdx.x; e < heads * N; e += 256) {
-    const int h = e / N, n = e % N, g = h / per;
-    const int64_t at = t * heads * N + e;
-    qf[at] = load_f32(row + heads * dv + (groups + g) * N + n);
-    kf[at] = static_cast<float>(steps[h] * static_cast<Acc>(load_f32(row + heads * dv + g * N + n)));
-    decay[at] = static_cast<float>(keeps[h]);
-  }
-  for (int e = threadIdx.x; e < heads * dv; e += 256) vf[t * heads * dv + e] = load_f32(row + e);
+  for (int j = 0; j < kConvMaxKeep; ++j)
+    if (j < keep) st[static_cast<int64_t>(j) * width + c] = j + 1 < keep ? kept[j + 1] : mine;
+  acc = acc / (static_cast<Acc>(1) + exp(-acc));
+  store_f32(xbc + t * xbc_stride + c, static_cast<float>(acc));
 }
 
 }  // namespace alofa
@@ -237,24 +211,6 @@ extern "C" int alofa_rms_pair_add_norm(float* residual, const float* a, const fl
   else if (normed == nullptr || normed_dtype == kF32) rms_pair_add_norm_kernel<float, float><<<grid, 256, 0, stream>>>(residual, a, wa, sa, b, wb, sb, scale, width, eps, static_cast<float*>(normed), nw, norm_eps);
   else rms_pair_add_norm_kernel<bf16_t, float><<<grid, 256, 0, stream>>>(residual, a, wa, sa, b, wb, sb, scale, width, eps, static_cast<bf16_t*>(normed), nw, norm_eps);
   return check_launch("rms_pair_add_norm");
-}
-
-extern "C" int alofa_ssd_step(void* xbc, int64_t xbc_stride, const void* raw, int64_t raw_stride, int dtype, const float* w, const float* bias, void* state,
-                              const int32_t* req_slot, int taps, float* qf, float* kf, float* vf, float* decay, const void* dt_raw, int64_t dt_stride,
-                              const float* dt_bias, const float* a_log, int64_t rows, int heads, int groups, int N, int dv, int exact, hipStream_t stream) {
-  ALOFA_REQUIRE(rows >= 0 && heads > 0 && groups > 0 && heads % groups == 0 && N > 0 && dv > 0, "ssd_step: bad sizes (heads=%d groups=%d state=%d dv=%d)", heads, groups, N, dv);
-  ALOFA_REQUIRE(taps >= 1 && taps - 1 <= kConvMaxKeep && (taps == 1 || state != nullptr), "ssd_step: 1 to %d taps, and a state for more than one", kConvMaxKeep + 1);
-  ALOFA_REQUIRE(!exact || dtype == kF32, "ssd_step: the exact path is float32");
-  if (rows == 0) return 0;
-  const size_t lds = 2 * static_cast<size_t>(heads) * sizeof(double);
-  ALOFA_REQUIRE(lds <= 32 * 1024, "ssd_step: %d heads", heads);
-#define ALOFA_SSDS(T, ACC) ssd_step_kernel<T, ACC><<<static_cast<unsigned>(rows), 256, lds, stream>>>(static_cast<T*>(xbc), xbc_stride, static_cast<const T*>(raw), raw_stride, w, bias, static_cast<T*>(state), \
-    req_slot, taps, qf, kf, vf, decay, static_cast<const T*>(dt_raw), dt_stride, dt_bias, a_log, heads, groups, N, dv)
-  if (exact) ALOFA_SSDS(float, double);
-  else if (dtype == kF32) ALOFA_SSDS(float, float);
-  else ALOFA_SSDS(bf16_t, float);
-#undef ALOFA_SSDS
-  return check_launch("ssd_step");
 }
 
 extern "C" int alofa_conv_bias_act(void* out, int64_t out_stride, int out_dtype, const void* x, int64_t x_stride, int x_dtype, const float* w, const float* bias,
@@ -320,4 +276,26 @@ extern "C" int alofa_rms_pair_sum(float* out, const float* a, const float* wa, f
   if (exact) rms_pair_sum_kernel<double><<<static_cast<unsigned>(rows), 256, 0, stream>>>(out, a, wa, sa, b, wb, sb, width, eps);
   else rms_pair_sum_kernel<float><<<static_cast<unsigned>(rows), 256, 0, stream>>>(out, a, wa, sa, b, wb, sb, width, eps);
   return check_launch("rms_pair_sum");
+}
+
+// The convolution (bias, silu) with its state's step for single rows, then the operands: two launches where rows of any number take three.
+// (All of it in one launch, a block per row that waits for its own row between the two halves, was measured and is slower: 18 us against the
+// 14 us of the three launches at eight rows of 2,560 channels; the two launches take 10.)
+extern "C" int alofa_ssd_step(void* xbc, int64_t xbc_stride, const void* raw, int64_t raw_stride, int dtype, const float* w, const float* bias, void* state,
+                              const int32_t* req_slot, int taps, float* qf, float* kf, float* vf, float* decay, const void* dt_raw, int64_t dt_stride,
+                              const float* dt_bias, const float* a_log, int64_t rows, int heads, int groups, int N, int dv, int exact, hipStream_t stream) {
+  ALOFA_REQUIRE(rows >= 0 && heads > 0 && groups > 0 && heads % groups == 0 && N > 0 && dv > 0, "ssd_step: bad sizes (heads=%d groups=%d state=%d dv=%d)", heads, groups, N, dv);
+  ALOFA_REQUIRE(taps >= 1 && taps - 1 <= kConvMaxKeep && (taps == 1 || state != nullptr), "ssd_step: 1 to %d taps, and a state for more than one", kConvMaxKeep + 1);
+  ALOFA_REQUIRE(!exact || dtype == kF32, "ssd_step: the exact path is float32");
+  if (rows == 0) return 0;
+  const int width = heads * dv + 2 * groups * N;
+  const dim3 grid((width + 255) / 256, static_cast<unsigned>(rows));
+#define ALOFA_SSDS(T, ACC) conv_step_kernel<T, ACC><<<grid, 256, 0, stream>>>(static_cast<T*>(xbc), xbc_stride, static_cast<const T*>(raw), raw_stride, w, bias, static_cast<T*>(state), \
+    req_slot, width, taps)
+  if (exact) ALOFA_SSDS(float, double);
+  else if (dtype == kF32) ALOFA_SSDS(float, float);
+  else ALOFA_SSDS(bf16_t, float);
+#undef ALOFA_SSDS
+  if (int e = check_launch("ssd_step")) return e;
+  return alofa_ssd_operands(qf, kf, vf, decay, xbc, xbc_stride, dt_raw, dt_stride, dtype, dt_bias, a_log, rows, heads, groups, N, dv, exact, stream);
 }

@@ -1913,7 +1913,7 @@ def rms_pair_add_norm(residual: torch.Tensor, a: torch.Tensor, wa: torch.Tensor,
 def ssd_step(xbc: torch.Tensor, raw: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], state: Optional[torch.Tensor], rows: RowsOfRequests, qf: torch.Tensor,
              kf: torch.Tensor, vf: torch.Tensor, decay: torch.Tensor, dt_raw: torch.Tensor, dt_bias: torch.Tensor, a_log: torch.Tensor, heads: int, groups: int,
              n_state: int, dv: int, exact: bool = False) -> None:
-    """``conv_bias_act`` (with silu), ``conv_keep`` and ``ssd_operands`` in one launch, for a step in which every request brings one row."""
+    """``conv_bias_act`` (with silu) and ``conv_keep`` in one launch, then ``ssd_operands``, for a step in which every request brings one row."""
     T, width = raw.shape
     taps = w.shape[1]
     _gpu("xbc", xbc, raw.dtype, 2), _gpu("raw", raw, None, 2), _gpu("w", w, torch.float32, 2), _contig("w", w)

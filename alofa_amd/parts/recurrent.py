@@ -328,7 +328,7 @@ class StateSpace(RecurrentMixer):
         qf, kf = ctx.scratch("memory_q", (T, H * N), torch.float32), ctx.scratch("memory_k", (T, H * N), torch.float32)
         vf, decay = ctx.scratch("memory_v", (T, inner), torch.float32), ctx.scratch("recurrent_decay", (T, H * N), torch.float32)
         tail = ctx.state((entry, k + 1)) if self.taps > 1 else None
-        if rows.offsets is None:      # single rows (decoding): the convolution, its state's step and the operands are one launch
+        if rows.offsets is None:      # single rows (decoding): the convolution and its state's step are one launch
             ops.ssd_step(xbc, raw, self.conv_w, self.conv_b, tail, rows, qf, kf, vf, decay, dt, self.dt_bias, self.a_log, H, self.groups, N, dv, exact)
         else:
             if tail is not None:

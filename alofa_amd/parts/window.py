@@ -17,7 +17,8 @@ reads key/value head h // (heads / kv_heads)). Then, each optional and chosen by
   sink        a number per head whose exponential joins the softmax's denominator (no key, no value).
   gate        "channel": the heads' outputs times sigmoid(Wg x), one gate per output channel; "head": one gate per head.
 
-Then the output projection. Scores, the softmax, norms and angles are float32 (float64 sums in the exact path).
+Then the output projection. Scores, the softmax, norms and angles are float32 (float64 sums in the exact path); on the matrix cores every
+softmax weight meets the values as two bfloat16 numbers, its rounding and what the rounding took away.
 
 The pages hold keys as [kv_head, slot, d] and values transposed, [kv_head, d, slot], as the other attention parts' (heads of unequal key and
 value size are widened with zero rows to one size d, so that the matrix-core kernels can read them). The pooled blocks live in pages of their own
@@ -196,14 +197,15 @@ class WindowAttention(Mixer):
         plan = ctx.memo("gqa_attention.rows", lambda: RowPlan(ctx))
         common = (self.heads, self.kv_heads, self.d, self.window, self.scale)
         if plan.long_runs is not None:
-            tiles, share, rows = plan.tiles(self.heads, self.kv_heads, self.d, self.window)
-            ops.attention_prefill(attn, q, kv.k, kv.v, kv.block_table, tiles, *common, share=share, rows=rows)
+            # (softmax weights are 32-bit numbers in this part: the form of the kernel that takes them as two bfloat16 numbers each)
+            tiles, share, rows = plan.tiles(self.heads, self.kv_heads, self.d, self.window, plain=True)
+            ops.attention_prefill(attn, q, kv.k, kv.v, kv.block_table, tiles, *common, share=share, rows=rows, fine_weights=True)
         if plan.n_short:
             floats = ops.decode_scratch_floats(plan.n_short, self.heads, self.kv_heads, self.d, ctx.max_context, self.window)
             partial = ctx.scratch("attn_partial", (floats,), torch.float32) if floats else None
             one_each = ctx.max_q_len == 1 and plan.short_rows is None and plan.long_runs is None
             ops.attention_decode(attn, q, kv.k, kv.v, kv.block_table, None if one_each else ctx.req_of_token, ctx.positions, *common,
-                                 ctx.max_context, partial, rows=plan.short_rows)
+                                 ctx.max_context, partial, rows=plan.short_rows, fine_weights=True)
 
     def forward(self, ctx, where, x, residual, out=None):
         T, exact = residual.shape[0], self.rt.exact
