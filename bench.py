@@ -556,10 +556,10 @@ def ludelorn_sizes(width, heads, dim, ff, layers, vocab=32000):
     beside a recurrence, dense feed-forwards), at equal width, heads, layers and feed-forward."""
     kv = max(1, heads // 4)
     left = {"heads": heads, "kv_heads": kv, "dim": dim, "vdim": dim, "scale": dim ** -0.5, "mask": {"size": 1024},
-            "rot": {"dims": dim, "base": 1000000.0, "scaling": {"factor": 4.0, "original": 4096, "fast": 32.0, "slow": 1.0}}}
+            "rot": {"dims": dim, "base": 250000.0, "scaling": {"factor": 4.0, "original": 4096, "fast": 16.0, "slow": 2.0}}}
     right = {"heads": heads, "vdim": dim, "state": dim, "groups": max(1, heads // 8), "conv": 4, "norm_groups": max(1, heads // 8)}
     kinds = [("parallel", {"left": left, "right": right}),
-             ("attention", {"heads": heads, "kv_heads": kv, "dim": dim, "vdim": dim, "scale": dim ** -0.5, "mask": {"size": 512, "pool": 16}, "rot": {"dims": dim // 2, "base": 500000.0}}),
+             ("attention", {"heads": heads, "kv_heads": kv, "dim": dim, "vdim": dim, "scale": dim ** -0.5, "mask": {"size": 512, "pool": 16}, "rot": {"dims": dim // 2, "base": 100000.0}}),
              ("parallel", {"left": left, "right": right}),
              ("attention_2", {"heads": heads, "kv_heads": kv, "dim": dim, "vdim": dim, "scale": 8.0 / dim, "mask": {"size": 512}, "bias_max": 512.0, "bias_rows": 32})]
     lud = {"architecture": "Ludelorn", "vocab": vocab, "width": width, "norm": {"eps": 1e-6}, "embedding": {"scale": 1.0},

@@ -99,7 +99,7 @@ def test_what_every_layer_keeps():
 
 @pytest.mark.parametrize("rot", [
     {"base": 10000.0, "dims": 8, "scaling": {"factor": 4.0, "original": 64, "fast": 8.0, "slow": 2.0}},
-    {"base": 1000000.0, "dims": 32, "scaling": {"factor": 2.0, "original": 2048, "fast": 32.0, "slow": 1.0}},
+    {"base": 250000.0, "dims": 32, "scaling": {"factor": 3.0, "original": 1024, "fast": 16.0, "slow": 2.0}},
     {"base": 777.0, "dims": 6},
     {"base": 50.0, "dims": 16, "scaling": {"factor": 8.0, "original": 16, "fast": 2.0, "slow": 1.5}},
 ])
@@ -131,7 +131,7 @@ def test_the_table_of_angles_is_the_plain_one(rot, pairing):
 
 def test_the_bias_rows_are_the_plain_ones():
     from alofa_amd.parts.window import distance_buckets
-    for rows, far in ((32, 120.0), (8, 14.0), (6, 5.0), (2, 3.0), (16, 30.0), (7, 100.5)):
+    for rows, far in ((24, 90.0), (8, 14.0), (6, 5.0), (2, 3.0), (16, 30.0), (7, 100.5)):
         upto = int(math.ceil(far)) + 3
         assert distance_buckets(rows, far, upto) == [pl.distance_bucket(n, rows, far) for n in range(upto)]
         assert pl.distance_bucket(10 ** 6, rows, far) == rows - 1 == distance_buckets(rows, far, upto)[-1]
