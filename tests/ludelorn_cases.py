@@ -65,6 +65,14 @@ LUDELORN = {
         (_pooled(2, 1, 16, 16, 4, 64.0, 0.3, 4, pool=1), None),
         (_parallel(_left(1, 1, 32, 16, 2, 10.0, 0.2, 2), _right(1, 24, 20, 1, 1, 3)), 40),
         (_biased(1, 1, 8, 0.5, 300, 32, 120.0), None)]),
+    # wider, in yet another order: heads of 80 and 112 channels (widened to 128), of 64 and 48 (to 64), of 48; a bias that reaches beyond its window; five groups of B and C;
+    # blocks of nine
+    "E": _config(401, 320, 1e-6, 4.0, [
+        (_biased(6, 3, 48, 0.2, 130, 20, 200.0), 512),
+        (_parallel(_left(6, 2, 80, 112, 64, 300000.0, 0.11, 100, scaling=(3.0, 512, 16.0, 2.0)), _right(10, 40, 24, 5, 3, 4)), 448),
+        (_pooled(4, 4, 64, 48, 32, 20000.0, 0.125, 70, pool=9), 512),
+        (_pooled(8, 2, 32, 32, 32, 7000.0, 0.2, 48, pool=20), None),
+        (_parallel(_left(4, 4, 96, 96, 48, 150000.0, 0.1, 160), _right(5, 64, 32, 1, 4, 1)), 384)]),
 }
 
 

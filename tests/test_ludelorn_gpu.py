@@ -15,7 +15,7 @@ from plain import ludelorn as pl
 pytestmark = pytest.mark.gpu
 
 DTYPES = ["float32", "bfloat16"]
-LENGTHS = {"A": 110, "B": 90, "C": 130, "D": 80}
+LENGTHS = {"A": 110, "B": 90, "C": 130, "D": 80, "E": 260}
 
 
 @pytest.fixture(scope="module")
@@ -142,6 +142,17 @@ def test_unequal_requests_together_with_slots_and_pages_used_again(ludelorn_dirs
             compare(got[req], ludelorn_dirs[name], ids, dtype, f"{name} mixed {req}")
     else:
         compare_together([(got[req], ids) for req, ids in requests.items()], ludelorn_dirs[name], dtype, f"{name} mixed")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_a_long_prompt_and_long_decoding(ludelorn_dirs, dtype):
+    """Hundreds of tokens through the wider model: several tiles of keys and of blocks a row, decoding across page borders, windows' and blocks' edges."""
+    from alofa_amd.replay import Replayer
+    ids = ids_of("E", 700, seed=31)
+    r = Replayer(ludelorn_dirs["E"], dtype, 1408, max_requests=2)
+    compare(collect(r, portions("p", ids, sizes=(300, 2, 150, 17, 3, 64, 5)))["p"], ludelorn_dirs["E"], ids, dtype, "long, portions")
+    compare(collect(r, bulk_and_tail("t", ids, tail=120))["t"], ludelorn_dirs["E"], ids, dtype, "long, decoding")
+    r.cache.check()
 
 
 def test_a_slot_used_again_starts_from_nothing(replayers, ludelorn_dirs):
@@ -299,6 +310,23 @@ def test_an_old_token_in_the_state(tmp_path, dtype):
     compare(collect(r, bulk_and_tail("t", ids, tail=60))["t"], d, ids, dtype, "old token, decoding")
     cfg, w = plain_model(str(d))
     assert np.abs(pl.forward_logits(w, cfg, ids)[-1] - pl.forward_logits(w, cfg, ids[150:])[-1]).max() > 0.02      # (the first half still counts at the end)
+
+
+@pytest.mark.parametrize("size", [80, 112, 256])
+def test_head_sizes_the_kernels_share_out_differently(tmp_path, size):
+    """Heads of one size in steps of sixteen that the engine's prefill kernel is not built for (80, 112: portions of prompts of a plain window then take this
+    part's matrix-core kernel, single tokens the engine's decode kernel, over the same pages), and the largest: portions, then decoding, in bfloat16."""
+    from alofa_amd.replay import Replayer
+
+    def change(cfg):
+        for l in cfg["layers"]:
+            m = l["mixer"]["left"] if l["type"] == "parallel" else l["mixer"]
+            m.update(dim=size, vdim=size, scale=(3.0 if l["type"] == "attention_2" else 1.0) / size ** 0.5)
+    d = _variant(LUDELORN["C"], tmp_path / "sizes", 800 + size, change)
+    ids = ids_of("C", 120, seed=29)
+    r = Replayer(d, "bfloat16", 256, max_requests=2)
+    compare(collect(r, portions("p", ids, sizes=(47, 2, 16, 17, 3, 15)))["p"], d, ids, "bfloat16", f"heads of {size}, portions")
+    compare(collect(r, bulk_and_tail("t", ids, tail=50))["t"], d, ids, "bfloat16", f"heads of {size}, decoding")
 
 
 def test_which_kernels_serve_which_layer(replayers, ludelorn_dirs, monkeypatch):
