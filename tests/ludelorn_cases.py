@@ -59,8 +59,8 @@ LUDELORN = {
         (_pooled(2, 1, 64, 64, 64, 1000.0, 0.12, 17), 48),
         (_pooled(2, 2, 48, 48, 24, 300.0, 0.15, 19, pool=3), None)]),
     # edges: a window of one key under a sink; blocks of one token (everything behind the window stays visible, token by token); a convolution of one tap;
-    # one head; a bias table of two rows
-    "D": _config(97, 48, 1e-5, 2.0, [
+    # one head; a bias table of two rows; a width that is no multiple of eight
+    "D": _config(97, 52, 1e-5, 2.0, [
         (_biased(2, 2, 24, 0.2, 1, 2, 3.0), 32),
         (_pooled(2, 1, 16, 16, 4, 64.0, 0.3, 4, pool=1), None),
         (_parallel(_left(1, 1, 32, 16, 2, 10.0, 0.2, 2), _right(1, 24, 20, 1, 1, 3)), 40),
