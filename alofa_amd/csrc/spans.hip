@@ -276,9 +276,9 @@ __global__ void __launch_bounds__(256) span_attention_kernel(T* __restrict__ out
   }
 }
 
-// ---- the matrix-core kernel: a block of four or eight wavefronts per (16 rows of one request, head), bfloat16
-// The wavefronts take the tiles of keys in turn (a row's chain of dependent tiles is as many times shorter) and their running states meet
-// in LDS at the end, combined in wavefront order.
+// ---- the matrix-core kernel: a wavefront, or a block of wavefronts, per (16 rows of one request, head), bfloat16
+// Where a block's wavefronts share a head they take the tiles of keys in turn (a row's chain of dependent tiles is as many times shorter) and
+// their running states meet in LDS at the end, combined in wavefront order.
 // Both products are taken transposed (v_mfma_f32_16x16x32_bf16; lane l: A row and B column l % 16, reduction slots 8 (l / 16) .. + 7,
 // D column l % 16 and rows 4 (l / 16) .. + 3), so a lane stays with one query row throughout:
 //   S^T[key, q] = K[key, :] . Q[q, :]       A = keys straight from the pages (16 bytes a lane), B = queries (registers)
@@ -309,16 +309,20 @@ struct SpanFastArgs {
   int gate_kind;
 };
 
-template <int DT, int NW>
+template <int DT, int NW, bool kDeal>
 __global__ void __launch_bounds__(64 * NW) span_attention_mfma_kernel(bf16_t* __restrict__ out, const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_cache,
                                                                   const bf16_t* __restrict__ v_cache, const bf16_t* __restrict__ pk, const bf16_t* __restrict__ pv,
                                                                   const bf16_t* __restrict__ gate, SpanFastArgs a) {
   constexpr int d = DT * 16, DS = (d + 31) / 32;
   constexpr float kLow = -1e30f;
-  __shared__ float others_acc[NW - 1][DT][kWave][4];      // what the other wavefronts hand to the first: their sums, ...
-  __shared__ float others_ml[NW - 1][2][kWave];           // ... maxima and weights' sums
-  const int lane = threadIdx.x % kWave, col = lane % 16, grp = lane / 16, wave = threadIdx.x / kWave;
-  const int h = blockIdx.y;
+  // kDeal: the block's wavefronts share one head and deal its tiles of keys out; else every wavefront has a head of its own (NW heads a block, neighbours of one
+  // key head: they walk the same tiles at about the same time, and what one has fetched the others find in the caches)
+  __shared__ float others_acc[kDeal ? NW - 1 : 1][kDeal ? DT : 1][kDeal ? kWave : 1][4];      // what the other wavefronts hand to the first: their sums, ...
+  __shared__ float others_ml[kDeal ? NW - 1 : 1][2][kDeal ? kWave : 1];                       // ... maxima and weights' sums
+  const int lane = threadIdx.x % kWave, col = lane % 16, grp = lane / 16, wave = kDeal ? threadIdx.x / kWave : 0;
+  const int h = kDeal ? blockIdx.y : blockIdx.y * NW + threadIdx.x / kWave;
+  constexpr int kStep = kDeal ? 32 * NW : 32;
+  if (!kDeal && h >= a.heads) return;
   const int g = h / (a.heads / a.kv_heads), S = 1 << a.bs_shift;
   int r, row0, n;
   if (a.tiles) {
@@ -380,7 +384,7 @@ __global__ void __launch_bounds__(64 * NW) span_attention_mfma_kernel(bf16_t* __
   };
 
   // ---- the window's tokens
-  for (int t0 = (lo / 32) * 32 + 32 * wave; t0 <= p_last; t0 += 32 * NW) {
+  for (int t0 = (lo / 32) * 32 + 32 * wave; t0 <= p_last; t0 += kStep) {
     span_f32x4 sc[2];
     bool seen[2][4];
 #pragma unroll
@@ -432,7 +436,7 @@ __global__ void __launch_bounds__(64 * NW) span_attention_mfma_kernel(bf16_t* __
       page = ptab[first >> a.bs_shift];
       place = (first & (S - 1)) / a.P;
     };
-    for (int e0 = 32 * wave; e0 < n_blk_tile; e0 += 32 * NW) {
+    for (int e0 = 32 * wave; e0 < n_blk_tile; e0 += kStep) {
       span_f32x4 sc[2];
       bool seen[2][4];
 #pragma unroll
@@ -472,6 +476,7 @@ __global__ void __launch_bounds__(64 * NW) span_attention_mfma_kernel(bf16_t* __
   }
 
   float total = rows_sum(l);
+  if constexpr (kDeal) {
   if (wave > 0) {
     others_ml[wave - 1][0][lane] = m;
     others_ml[wave - 1][1][lane] = total;
@@ -491,6 +496,7 @@ __global__ void __launch_bounds__(64 * NW) span_attention_mfma_kernel(bf16_t* __
     for (int o = 0; o < DT; ++o)
 #pragma unroll
       for (int x = 0; x < 4; ++x) acc[o][x] = acc[o][x] * mine + others_acc[w][o][lane][x] * theirs;
+  }
   }
   if (a.sink) {
     const float sk = a.sink[h], m_f = fmaxf(m, sk), alpha = __expf(m - m_f);
@@ -607,13 +613,15 @@ extern "C" int alofa_span_attention(void* out, int64_t out_stride, const void* q
 template <int DT>
 static void launch_span_mfma(dim3 grid, hipStream_t stream, void* out, const void* q, const void* k_cache, const void* v_cache, const void* pk, const void* pv, const void* gate,
                              const SpanFastArgs& a) {
-  // (single rows, where blocks are few: eight wavefronts where their states fit the LDS a block may name; runs of rows: four, 78 against 91 us a layer of a 2,048-token prompt)
-  if (DT <= 8 && a.tiles == nullptr)
-    span_attention_mfma_kernel<DT, (DT <= 8 ? 8 : 4)><<<grid, 64 * 8, 0, stream>>>(static_cast<bf16_t*>(out), static_cast<const bf16_t*>(q), static_cast<const bf16_t*>(k_cache), static_cast<const bf16_t*>(v_cache),
-                                                                            static_cast<const bf16_t*>(pk), static_cast<const bf16_t*>(pv), static_cast<const bf16_t*>(gate), a);
-  else
-    span_attention_mfma_kernel<DT, 4><<<grid, 256, 0, stream>>>(static_cast<bf16_t*>(out), static_cast<const bf16_t*>(q), static_cast<const bf16_t*>(k_cache), static_cast<const bf16_t*>(v_cache),
-                                                                static_cast<const bf16_t*>(pk), static_cast<const bf16_t*>(pv), static_cast<const bf16_t*>(gate), a);
+  // Single rows, where blocks are few: a block per row and head, its eight wavefronts (four for heads wider than 128 channels: their states must fit the LDS a block
+  // may name) deal the tiles of keys out. Runs of rows, where blocks are many: four heads a block, a wavefront each (a layer of a 2,048-token prompt at 16 heads of 128:
+  // 78 us, against 79 with four and 91 with eight wavefronts dealing a head's tiles out, and no LDS).
+#define ALOFA_SPAN_LAUNCH(NW, DEAL, GRID) span_attention_mfma_kernel<DT, NW, DEAL><<<GRID, 64 * NW, 0, stream>>>(static_cast<bf16_t*>(out), static_cast<const bf16_t*>(q), \
+    static_cast<const bf16_t*>(k_cache), static_cast<const bf16_t*>(v_cache), static_cast<const bf16_t*>(pk), static_cast<const bf16_t*>(pv), static_cast<const bf16_t*>(gate), a)
+  if (a.tiles != nullptr) ALOFA_SPAN_LAUNCH(4, false, dim3(grid.x, (a.heads + 3) / 4));
+  else if (DT <= 8) ALOFA_SPAN_LAUNCH((DT <= 8 ? 8 : 4), true, grid);
+  else ALOFA_SPAN_LAUNCH(4, true, grid);
+#undef ALOFA_SPAN_LAUNCH
 }
 
 // bfloat16 on the matrix cores: heads of d = dv channels in steps of 16, pages of a power of two of at least 8 tokens, rows 16-byte aligned.

@@ -101,14 +101,28 @@ __global__ void __launch_bounds__(256) ssd_finish_kernel(T* __restrict__ out, in
     const Acc g = static_cast<Acc>(load_f32(z + t * z_stride + c));
     return y * (g / (static_cast<Acc>(1) + exp(-g)));
   };
+  // (parts of up to 2,048 channels wait in registers between the sum of squares and the scaling; wider ones are formed twice)
+  constexpr int kOwn = 8;
+  Acc own[kOwn];
   Acc ss = 0;
-  for (int c = c0 + threadIdx.x; c < c0 + span; c += 256) {
+#pragma unroll
+  for (int n = 0; n < kOwn; ++n) {
+    const int c = c0 + threadIdx.x + n * 256;
+    own[n] = c < c0 + span ? value(c) : static_cast<Acc>(0);
+    ss += own[n] * own[n];
+  }
+  for (int c = c0 + threadIdx.x + kOwn * 256; c < c0 + span; c += 256) {
     const Acc y = value(c);
     ss += y * y;
   }
   ss = block_sum<Acc, 256>(ss, scratch);
   const Acc inv = static_cast<Acc>(1) / sqrt(ss / static_cast<Acc>(span) + static_cast<Acc>(eps));
-  for (int c = c0 + threadIdx.x; c < c0 + span; c += 256)
+#pragma unroll
+  for (int n = 0; n < kOwn; ++n) {
+    const int c = c0 + threadIdx.x + n * 256;
+    if (c < c0 + span) store_f32(out + t * out_stride + c, static_cast<float>(own[n] * inv * static_cast<Acc>(weight[c])));
+  }
+  for (int c = c0 + threadIdx.x + kOwn * 256; c < c0 + span; c += 256)
     store_f32(out + t * out_stride + c, static_cast<float>(value(c) * inv * static_cast<Acc>(weight[c])));
 }
 
