@@ -387,6 +387,16 @@ __global__ void __launch_bounds__(64 * NW) span_attention_mfma_kernel(bf16_t* __
   for (int t0 = (lo / 32) * 32 + 32 * wave; t0 <= p_last; t0 += kStep) {
     span_f32x4 sc[2];
     bool seen[2][4];
+    // the tile's values are asked for first: they are on their way while the scores are formed (they do not depend on them)
+    uint2 vraw[DT][2];
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      int j = t0 + 16 * u + 4 * grp;      // (four keys of one page; clamped to a run whose page is held)
+      j = j < (lo & ~3) ? (lo & ~3) : (j > (p_last & ~3) ? (p_last & ~3) : j);
+      const bf16_t* vrow = v_cache + ((static_cast<int64_t>(tab[j >> a.bs_shift]) * a.kv_heads + g) * d + col) * S + (j & (S - 1));
+#pragma unroll
+      for (int o = 0; o < DT; ++o) vraw[o][u] = *reinterpret_cast<const uint2*>(vrow + static_cast<int64_t>(o) * 16 * S);
+    }
 #pragma unroll
     for (int u = 0; u < 2; ++u) {
       int key = t0 + 16 * u + col;      // (the key this lane fetches for the first product: clamped to one whose page is held)
@@ -410,18 +420,9 @@ __global__ void __launch_bounds__(64 * NW) span_attention_mfma_kernel(bf16_t* __
       }
     }
     softmax_step(sc, seen, [&](int o) {
-      span_bf16x8 vf;
-#pragma unroll
-      for (int u = 0; u < 2; ++u) {
-        int j = t0 + 16 * u + 4 * grp;      // (four keys of one page; clamped to a run whose page is held)
-        j = j < (lo & ~3) ? (lo & ~3) : (j > (p_last & ~3) ? (p_last & ~3) : j);
-        const bf16_t* vrow = v_cache + ((static_cast<int64_t>(tab[j >> a.bs_shift]) * a.kv_heads + g) * d + o * 16 + col) * S + (j & (S - 1));
-        const uint2 four = *reinterpret_cast<const uint2*>(vrow);
-        const uint32_t two[2] = {four.x, four.y};
-#pragma unroll
-        for (int x = 0; x < 4; ++x) vf[4 * u + x] = __builtin_bit_cast(__bf16, static_cast<uint16_t>(two[x / 2] >> (16 * (x % 2))));
-      }
-      return vf;
+      typedef uint32_t span_u32x4 __attribute__((ext_vector_type(4)));
+      const span_u32x4 raw = {vraw[o][0].x, vraw[o][0].y, vraw[o][1].x, vraw[o][1].y};
+      return __builtin_bit_cast(span_bf16x8, raw);
     });
   }
 
