@@ -17,7 +17,7 @@ Mixers by ``type``:
                channels with ``state`` channels of state each, B and C in ``groups`` groups, a convolution of ``conv`` taps, its gated read-out normed
                in ``norm_groups`` parts. The result is half the sum of the two, each through an RMS norm over the width (``left.out``, ``right.out``).
   attention    heads as above; queries and keys through an RMS norm over their whole projection (``q.norm``, ``k.norm``), then turned on their first
-               ``rot.dims`` channels (pairs (2i, 2i + 1)); a row sees the last ``mask.size`` keys and, behind them, the mean key and value of every whole
+               ``rot.dims`` channels (pairs (2i, 2i + 1); a ``rot.scaling`` is applied as on the left); a row sees the last ``mask.size`` keys and, behind them, the mean key and value of every whole
                block of ``mask.pool`` tokens; a sigmoid gate per output channel.
   attention_2  no ``v`` projection (a token's value is its key as projected) and no positions; queries and keys divided by their root mean square
                per head; the score gets ``rel``[bucket(distance), head] added (the table's rows: one per distance up to half of them, then evenly in the
@@ -50,15 +50,13 @@ def _heads(m: dict, where: str, values: bool = True) -> dict:
     return out
 
 
-def _rot(m: dict, dim: int, where: str, scaling: bool) -> dict:
+def _rot(m: dict, dim: int, where: str) -> dict:
     rot = _get(m, "rot", dict, where)
     r = {"base": _get(rot, "base", float, where), "dims": _get(rot, "dims", int, where)}
     _positive(where, base=r["base"], dims=r["dims"])
     if r["dims"] % 2 or r["dims"] > dim:
         raise AlofaError("parse", "rot.dims is even and at most the head's size", f"dims={r['dims']} dim={dim} config={where}")
     if rot.get("scaling") is not None:
-        if not scaling:
-            raise AlofaError("unsupported", "this mixer's positions are not stretched", f"config={where}")
         r["scaling"] = {k: _get(rot["scaling"], k, float, where) for k in ("factor", "original", "fast", "slow")}
         _positive(where, **r["scaling"])
     return r
@@ -66,7 +64,7 @@ def _rot(m: dict, dim: int, where: str, scaling: bool) -> dict:
 
 def _left(m: dict, where: str) -> dict:
     out = _heads(m, where)
-    out["rot"] = _rot(m, out["dim"], where, scaling=True)
+    out["rot"] = _rot(m, out["dim"], where)
     return out
 
 
@@ -83,7 +81,7 @@ def _mixer(kind: str, m: dict, where: str) -> dict:
         return {"left": _left(_get(m, "left", dict, where), where + " left"), "right": _right(_get(m, "right", dict, where), where + " right")}
     if kind == "attention":
         out = _heads(m, where)
-        out["rot"] = _rot(m, out["dim"], where, scaling=False)
+        out["rot"] = _rot(m, out["dim"], where)
         if m["mask"].get("pool") is not None:
             out["mask"]["pool"] = _get(m["mask"], "pool", int, where)
             _positive(where, pool=out["mask"]["pool"])
@@ -166,7 +164,7 @@ class LudelornConfig(ModelConfig):
         if kind == "attention":
             rot = m["rot"]
             return self._attention(m, pre, qk_norm="all", gate="channel", pool=m["mask"].get("pool"), position=PartSpec(
-                "rotary", {"theta": rot["base"], "head_dim": m["dim"], "dims": rot["dims"], "pairing": "neighbours", "frequencies": "direct"}))
+                "rotary", {"theta": rot["base"], "head_dim": m["dim"], "dims": rot["dims"], "pairing": "neighbours", "frequencies": "direct", "stretch": rot.get("scaling")}))
         if kind == "attention_2":
             return self._attention(m, pre, qk_norm="unit", gate="head", values_are_keys=True, sink=True, position=None,
                                    bias={"rows": m["bias_rows"], "far": m["bias_max"]})

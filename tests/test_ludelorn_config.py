@@ -68,7 +68,6 @@ def test_the_bias_table_is_sized_by_its_tensor(tmp_path):
     (lambda c: c["layers"][0]["mixer"]["left"]["rot"].update(dims=18), "rot.dims is even and at most"),
     (lambda c: c["layers"][0]["mixer"]["right"].update(groups=3), "groups divide the heads"),
     (lambda c: c["layers"][0]["mixer"]["right"].update(norm_groups=5), "groups divide the heads"),
-    (lambda c: c["layers"][1]["mixer"]["rot"].update(scaling={"factor": 2.0, "original": 64, "fast": 8.0, "slow": 1.0}), "not stretched"),
     (lambda c: c["layers"][1]["mixer"]["mask"].update(pool=0), "must be positive"),
     (lambda c: c["layers"][2]["mixer"].update(vdim=8), "values that are the keys"),
     (lambda c: c["layers"][2]["mixer"].pop("bias_max"), "lacks a required key"),
