@@ -51,12 +51,12 @@ def test_the_default_run_prints_one_line_with_the_agreed_keys():
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("design", ["tugalix", "rerupel"])
-def test_another_design_beside_the_closest_one_prints_a_line_per_point(design):
+@pytest.mark.parametrize("design,beside", [("tugalix", "qwen2"), ("rerupel", "qwen2"), ("ludelorn", "tugalix")])
+def test_another_design_beside_the_closest_one_prints_a_line_per_point(design, beside):
     rc, out, err = run_bench("--design", design, "--sizes", "256", "--prompt-tokens", "256", "--batches", "1,4", "--steps", "6", "--warmup", "2")
     assert rc == 0, err[-2000:]
     lines = [json.loads(line) for line in out.splitlines() if line.startswith("{")]
-    assert [(d["design"], d["point"], d.get("batch")) for d in lines] == [(m, p, b) for m in (design, "qwen2") for p, b in (("prefill", None), ("decode", 1), ("decode", 4))]
+    assert [(d["design"], d["point"], d.get("batch")) for d in lines] == [(m, p, b) for m in (design, beside) for p, b in (("prefill", None), ("decode", 1), ("decode", 4))]
     for d in lines:
         assert d["size"] == "256" and d["tok_s"] > 0
         if d["point"] == "prefill":
